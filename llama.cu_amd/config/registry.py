@@ -10,7 +10,7 @@ from __future__ import annotations
 import importlib
 import os
 from dataclasses import dataclass
-from typing import Any, Callable, Dict, Iterable, List, Tuple
+from typing import Any, Callable, Dict, Iterable, List, Optional, Tuple
 
 from .base import ConfigError, read_config_json
 
@@ -22,18 +22,20 @@ class Architecture:
     build_spec: Callable[[Any], Any]                    # typed configuration -> parts.ModelSpec
     ignored_tensors: Tuple[str, ...] = ()               # regular expressions: tensors that this architecture's files may
                                                         # carry beside the weights, which the loader passes over
+    complete_config: Any = None                         # (configuration, {tensor name: shape}) -> configuration: for a
+                                                        # design whose config.json leaves a size to the tensors' shapes
 
 
 _REGISTRY: Dict[str, Architecture] = {}
 
 
 def register_architecture(name: str, config_from_dict, build_spec, replace: bool = False,
-                          ignored_tensors: Iterable[str] = ()) -> None:
+                          ignored_tensors: Iterable[str] = (), complete_config=None) -> None:
     """``ignored_tensors``: regular expressions (matched from a tensor name's start) for tensors that files of this
     architecture may hold and that are no weights; every other tensor that the model does not expect is an error."""
     if name in _REGISTRY and not replace:
         raise ValueError(f"architecture {name!r} is already registered")
-    _REGISTRY[name] = Architecture(name, config_from_dict, build_spec, tuple(ignored_tensors))
+    _REGISTRY[name] = Architecture(name, config_from_dict, build_spec, tuple(ignored_tensors), complete_config)
 
 
 def registered_architectures() -> List[str]:
@@ -42,6 +44,8 @@ def registered_architectures() -> List[str]:
 
 def architecture_of(data: Dict[str, Any], where: str = "config.json") -> Architecture:
     names = data.get("architectures")
+    if names is None and isinstance(data.get("architecture"), str):
+        names = [data["architecture"]]              # some designs' files name the one architecture so
     if not isinstance(names, list) or not names or not isinstance(names[0], str):
         raise ConfigError(f"{where}: required key 'architectures' is missing or holds no name")
     arch = _REGISTRY.get(names[0])
@@ -80,8 +84,13 @@ def load_plugins_from_env() -> List[str]:
     return load_plugins(os.environ.get(PLUGINS_ENV, "").split(","))
 
 
-def load_config(folder: str):
-    """(architecture, typed configuration) of a model folder."""
+def load_config(folder: str, shapes: Optional[Dict[str, Tuple[int, ...]]] = None):
+    """(architecture, typed configuration) of a model folder.  ``shapes``: the shapes of the folder's tensors, for
+    an architecture whose configuration takes sizes from them (``complete_config``); without them such sizes
+    stay open, and building the model then says which."""
     data = read_config_json(folder)
     arch = architecture_of(data, where=f"{folder}/config.json")
-    return arch, arch.config_from_dict(data)
+    cfg = arch.config_from_dict(data)
+    if shapes is not None and arch.complete_config is not None:
+        cfg = arch.complete_config(cfg, shapes)
+    return arch, cfg

@@ -12,6 +12,7 @@
 //
 // head_slopes (may be null): a bias inside the scores that grows with the distance, for position
 // encodings of that kind: slope[h] * (j - p) is added to the scaled score of key j for the query at p.
+// dv: the values' head size (the keys' is dh); out is [n, nh * dv].
 #include "common.h"
 #include "kv_layout.h"
 
@@ -22,7 +23,7 @@ __global__ void __launch_bounds__(64)
 paged_attention_generic_kernel(const T *__restrict__ q, int q_stride, T *__restrict__ out, int out_stride,
                                const T *__restrict__ cache, const int *__restrict__ block_table, int max_pages,
                                const int *__restrict__ q_start, const int *__restrict__ ctx_len,
-                               const int *__restrict__ req_of_token, int nh, int nkvh, int dh, int page,
+                               const int *__restrict__ req_of_token, int nh, int nkvh, int dh, int dv, int page,
                                float scale, int window, const float *__restrict__ head_slopes) {
     const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
     const int r = req_of_token[t];
@@ -37,8 +38,8 @@ paged_attention_generic_kernel(const T *__restrict__ q, int q_stride, T *__restr
     __syncthreads();
 
     const int *bt = block_table + (size_t)r * max_pages;
-    const size_t page_elems = kv_page_elems(nkvh, dh, page);
-    const size_t v_base = (size_t)nkvh * dh * page + (size_t)kvh * dh * page;
+    const size_t page_elems = kv_page_elems(nkvh, dh, dv, page);
+    const size_t v_base = kv_value_offset(nkvh, kvh, 0, 0, dh, dv, page);
     float m = -INFINITY, l = 0.f;
     float o[MAX_HEAD_DIM / WAVE] = {0.f, 0.f, 0.f, 0.f};
 
@@ -75,7 +76,7 @@ paged_attention_generic_kernel(const T *__restrict__ q, int q_stride, T *__restr
 #pragma unroll
             for (int i = 0; i < MAX_HEAD_DIM / WAVE; ++i) {
                 const int d = lane + WAVE * i;
-                if (d < dh) o[i] += pp * to_f32(vp[(size_t)d * page]);
+                if (d < dv) o[i] += pp * to_f32(vp[(size_t)d * page]);
             }
         }
         __syncthreads();
@@ -84,7 +85,7 @@ paged_attention_generic_kernel(const T *__restrict__ q, int q_stride, T *__restr
 #pragma unroll
     for (int i = 0; i < MAX_HEAD_DIM / WAVE; ++i) {
         const int d = lane + WAVE * i;
-        if (d < dh) out[(size_t)t * out_stride + (size_t)h * dh + d] = from_f32<T>(o[i] * inv);
+        if (d < dv) out[(size_t)t * out_stride + (size_t)h * dv + d] = from_f32<T>(o[i] * inv);
     }
 }
 
@@ -96,17 +97,17 @@ paged_attention_generic_kernel(const T *__restrict__ q, int q_stride, T *__restr
 LCU_API int lcu_paged_attention_generic(const void *q, int q_stride, void *out, int out_stride, int type,
                                         const void *cache, const int *block_table, int max_pages,
                                         const int *q_start, const int *ctx_len, const int *req_of_token, int n,
-                                        int nh, int nkvh, int dh, int page, float scale, int window,
+                                        int nh, int nkvh, int dh, int dv, int page, float scale, int window,
                                         const float *head_slopes, hipStream_t stream) {
     if (n <= 0) return LCU_OK;
-    if (nh <= 0 || nkvh <= 0 || nh % nkvh || dh <= 0 || dh % 8 || dh > MAX_HEAD_DIM || page <= 0 || page % 8 ||
+    if (nh <= 0 || nkvh <= 0 || nh % nkvh || dh <= 0 || dh % 8 || dh > MAX_HEAD_DIM || dv <= 0 || dv > MAX_HEAD_DIM || page <= 0 || page % 8 ||
         max_pages <= 0 || window < 0 || nh > 65535)
         return LCU_BAD_ARGUMENT;
     dim3 grid(n, nh), block(WAVE);
     if (type == LCU_F32)
-        paged_attention_generic_kernel<float><<<grid, block, 0, stream>>>((const float *)q, q_stride, (float *)out, out_stride, (const float *)cache, block_table, max_pages, q_start, ctx_len, req_of_token, nh, nkvh, dh, page, scale, window, head_slopes);
+        paged_attention_generic_kernel<float><<<grid, block, 0, stream>>>((const float *)q, q_stride, (float *)out, out_stride, (const float *)cache, block_table, max_pages, q_start, ctx_len, req_of_token, nh, nkvh, dh, dv, page, scale, window, head_slopes);
     else if (type == LCU_BF16)
-        paged_attention_generic_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t *)q, q_stride, (bf16_t *)out, out_stride, (const bf16_t *)cache, block_table, max_pages, q_start, ctx_len, req_of_token, nh, nkvh, dh, page, scale, window, head_slopes);
+        paged_attention_generic_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t *)q, q_stride, (bf16_t *)out, out_stride, (const bf16_t *)cache, block_table, max_pages, q_start, ctx_len, req_of_token, nh, nkvh, dh, dv, page, scale, window, head_slopes);
     else
         return LCU_BAD_ARGUMENT;
     LCU_LAUNCH_CHECK();

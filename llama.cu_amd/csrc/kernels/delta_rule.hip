@@ -1,0 +1,192 @@
+// The generalised delta rule: a recurrent mixer whose state per head is a matrix S [dk, dv]
+// (key channel, value channel) in 32-bit.  For every token, with per key channel a decay w, a
+// removal rate a, the key k, its unit vector u = k / sqrt(sum(k^2) + 1e-6), the query r, and
+// per value channel v:
+//   S <- diag(w) S - (a * u) (u^T S) + k v^T        (both terms read the old S)
+//   o  = S^T r
+// Everything that enters the recurrence is 32-bit.  Three kernels:
+//   prep  (parallel over tokens and heads): w, a * u, u, k, r as 32-bit vectors;
+//           w = exp(-exp(-1/2) * sigmoid(w0 + W2 tanh(l))), l the row's low-rank projection,
+//           a = sigmoid(a_lin + a_bias);
+//   scan  (sequential over a request's tokens, parallel over requests, heads and value
+//           channels: column j of S depends on column j alone, so a lane owns a column and
+//           keeps it in registers from the request's first token of the step to its last);
+//   out   (parallel): o of each head divided by its root mean square, times a weight, times
+//           sigmoid(gate).
+// A token's result depends on the tokens before it in its request only, in an order of
+// operations that does not depend on how the request was cut into steps.
+#include "common.h"
+
+constexpr int MAX_RANK = 512;
+constexpr float DECAY_SCALE = 0.6065306597126334f;      // exp(-1/2)
+
+__device__ __forceinline__ float sigmoidf_(float z) { return 1.0f / (1.0f + expf(-z)); }
+
+// proj: [n, row_stride] rows that hold r, k, a_lin (dk per head each) and the low-rank
+// projection l (rank) at the given column offsets.  prep: [n, heads, 5, dk] 32-bit.
+template <class T>
+__global__ void delta_prep_kernel(const T *__restrict__ proj, int row_stride, int off_r, int off_k, int off_a, int off_l,
+                                  const float *__restrict__ w2, const float *__restrict__ w0,
+                                  const float *__restrict__ a_bias, float *__restrict__ prep, int heads, int dk, int rank) {
+    __shared__ float th[MAX_RANK];
+    __shared__ float scratch[16];
+    const int t = blockIdx.x, h = blockIdx.y;
+    const T *row = proj + (size_t)t * row_stride;
+    for (int i = threadIdx.x; i < rank; i += blockDim.x) th[i] = tanhf(to_f32(row[off_l + i]));
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < dk; i += blockDim.x) {
+        const float kk = to_f32(row[off_k + h * dk + i]);
+        ss += kk * kk;
+    }
+    ss = block_sum(ss, scratch);                 // (its barriers also make th visible)
+    const float inv = 1.0f / sqrtf(ss + 1e-6f);
+    float *out = prep + ((size_t)t * heads + h) * 5 * dk;
+    for (int i = threadIdx.x; i < dk; i += blockDim.x) {
+        const int c = h * dk + i;
+        float z = w0[c];
+        for (int j = 0; j < rank; ++j) z += w2[(size_t)c * rank + j] * th[j];
+        const float w = expf(-DECAY_SCALE * sigmoidf_(z));
+        const float a = sigmoidf_(to_f32(row[off_a + c]) + a_bias[c]);
+        const float kk = to_f32(row[off_k + c]);
+        const float u = kk * inv;
+        out[i] = w;
+        out[dk + i] = a * u;
+        out[2 * dk + i] = u;
+        out[3 * dk + i] = kk;
+        out[4 * dk + i] = to_f32(row[off_r + c]);
+    }
+}
+
+// One wave per (request, head, 64 value channels).  DK > 0: the column of S lives in DK
+// registers; DK == 0: any dk, the column stays in the state's memory.
+// state: [slots, heads, dk, dv]; o: [n, heads * dv] 32-bit.
+template <class T, int DK>
+__global__ void __launch_bounds__(64)
+delta_scan_kernel(const T *__restrict__ proj, int row_stride, int off_v, const float *__restrict__ prep,
+                  float *__restrict__ state, float *__restrict__ o, const int *__restrict__ q_start,
+                  const int *__restrict__ ctx_len, const int *__restrict__ state_slot, int heads, int dk_rt, int dv) {
+    const int dk = DK > 0 ? DK : dk_rt;
+    const int r = blockIdx.x, h = blockIdx.y, j = blockIdx.z * 64 + threadIdx.x;
+    const int t0 = q_start[r], t1 = q_start[r + 1];
+    const bool fresh = ctx_len[r] - (t1 - t0) == 0;          // the request's first token: the state starts at zero
+    const bool live = j < dv;
+    const int jj = live ? j : dv - 1;                        // lanes beyond dv compute along and store nothing
+    float *col = state + (((size_t)state_slot[r] * heads + h) * dk) * dv + jj;     // S[i][j] at col[i * dv]
+    __shared__ float vec[2][5 * (DK > 0 ? DK : 1)];
+    float S[DK > 0 ? DK : 1];
+    if (DK > 0) {
+#pragma unroll
+        for (int i = 0; i < DK; ++i) S[i] = fresh ? 0.f : col[(size_t)i * dv];
+    } else if (fresh && live) {
+        for (int i = 0; i < dk; ++i) col[(size_t)i * dv] = 0.f;
+    }
+    constexpr int PER_LANE = DK > 0 ? (5 * DK + 63) / 64 : 1;
+    float next[PER_LANE];
+    auto fetch = [&](int t) {
+        const float *p = prep + ((size_t)t * heads + h) * 5 * dk;
+#pragma unroll
+        for (int e = 0; e < PER_LANE; ++e) {
+            const int idx = e * 64 + threadIdx.x;
+            next[e] = idx < 5 * dk ? p[idx] : 0.f;
+        }
+    };
+    if (DK > 0 && t0 < t1) fetch(t0);
+    for (int t = t0; t < t1; ++t) {
+        const float v = to_f32(proj[(size_t)t * row_stride + off_v + h * dv + jj]);
+        float acc = 0.f;
+        if (DK > 0) {
+            float *cur = vec[(t - t0) & 1];
+#pragma unroll
+            for (int e = 0; e < PER_LANE; ++e) {
+                const int idx = e * 64 + threadIdx.x;
+                if (idx < 5 * DK) cur[idx] = next[e];
+            }
+            __syncthreads();
+            if (t + 1 < t1) fetch(t + 1);
+            const float *W = cur, *AU = cur + DK, *U = cur + 2 * DK, *K = cur + 3 * DK, *R = cur + 4 * DK;
+            float us = 0.f;
+#pragma unroll
+            for (int i = 0; i < DK; ++i) us += U[i] * S[i];
+#pragma unroll
+            for (int i = 0; i < DK; ++i) {
+                S[i] = W[i] * S[i] - AU[i] * us + K[i] * v;
+                acc += S[i] * R[i];
+            }
+        } else {
+            const float *p = prep + ((size_t)t * heads + h) * 5 * dk;
+            float us = 0.f;
+            for (int i = 0; i < dk; ++i) us += p[2 * dk + i] * col[(size_t)i * dv];
+            for (int i = 0; i < dk; ++i) {
+                const float s = p[i] * col[(size_t)i * dv] - p[dk + i] * us + p[3 * dk + i] * v;
+                if (live) col[(size_t)i * dv] = s;
+                acc += s * p[4 * dk + i];
+            }
+        }
+        if (live) o[(size_t)t * heads * dv + h * dv + j] = acc;
+    }
+    if (DK > 0 && live) {
+#pragma unroll
+        for (int i = 0; i < DK; ++i) col[(size_t)i * dv] = S[i];
+    }
+}
+
+// One wave per (token, head): out = o / rms(o) * weight * sigmoid(gate).
+template <class T>
+__global__ void __launch_bounds__(64)
+delta_out_kernel(const float *__restrict__ o, const T *__restrict__ proj, int row_stride, int off_g,
+                 const float *__restrict__ weight, T *__restrict__ out, int heads, int dv, float eps) {
+    const int t = blockIdx.x, h = blockIdx.y;
+    const float *oh = o + (size_t)t * heads * dv + h * dv;
+    float ss = 0.f;
+    for (int j = threadIdx.x; j < dv; j += 64) ss += oh[j] * oh[j];
+    const float f = rsqrtf(wave_sum(ss) / (float)dv + eps);
+    for (int j = threadIdx.x; j < dv; j += 64) {
+        const int c = h * dv + j;
+        const float g = sigmoidf_(to_f32(proj[(size_t)t * row_stride + off_g + c]));
+        out[(size_t)t * heads * dv + c] = from_f32<T>(oh[j] * f * weight[c] * g);
+    }
+}
+
+template <class T>
+static int delta_rule_t(const T *proj, int row_stride, int off_r, int off_k, int off_v, int off_g, int off_a, int off_l,
+                        const float *w2, const float *w0, const float *a_bias, const float *weight, float *prep,
+                        float *o, float *state, T *out, const int *q_start, const int *ctx_len, const int *state_slot,
+                        int n, int n_req, int heads, int dk, int dv, int rank, float eps, hipStream_t stream) {
+    int threads = ((dk > rank ? dk : rank) + 63) / 64 * 64;
+    if (threads > 256) threads = 256;
+    delta_prep_kernel<T><<<dim3(n, heads), dim3(threads), 0, stream>>>(proj, row_stride, off_r, off_k, off_a, off_l, w2, w0, a_bias, prep, heads, dk, rank);
+    LCU_LAUNCH_CHECK();
+    dim3 grid(n_req, heads, (dv + 63) / 64);
+#define SCAN(DK) delta_scan_kernel<T, DK><<<grid, dim3(64), 0, stream>>>(proj, row_stride, off_v, prep, state, o, q_start, ctx_len, state_slot, heads, dk, dv)
+    switch (dk) {
+    case 16: SCAN(16); break;
+    case 32: SCAN(32); break;
+    case 48: SCAN(48); break;
+    case 64: SCAN(64); break;
+    case 96: SCAN(96); break;
+    case 128: SCAN(128); break;
+    default: SCAN(0); break;
+    }
+#undef SCAN
+    LCU_LAUNCH_CHECK();
+    delta_out_kernel<T><<<dim3(n, heads), dim3(64), 0, stream>>>(o, proj, row_stride, off_g, weight, out, heads, dv, eps);
+    LCU_LAUNCH_CHECK();
+    return LCU_OK;
+}
+
+// proj: [n, row_stride] of `type`; the offsets are columns.  w2: [heads * dk, rank], w0, a_bias: [heads * dk],
+// weight: [heads * dv], all 32-bit.  prep: scratch [n, heads, 5, dk], o: scratch [n, heads * dv], both 32-bit.
+// state: [slots, heads, dk, dv] 32-bit.  out: [n, heads * dv] of `type`.
+LCU_API int lcu_delta_rule(const void *proj, int type, int row_stride, int off_r, int off_k, int off_v, int off_g,
+                           int off_a, int off_l, const float *w2, const float *w0, const float *a_bias,
+                           const float *weight, float *prep, float *o, float *state, void *out, const int *q_start,
+                           const int *ctx_len, const int *state_slot, int n, int n_req, int heads, int dk, int dv,
+                           int rank, float eps, hipStream_t stream) {
+    if (n <= 0 || n_req <= 0) return LCU_OK;
+    if (heads <= 0 || heads > 65535 || dk <= 0 || dv <= 0 || rank <= 0 || rank > MAX_RANK || dv > 64 * 65535) return LCU_BAD_ARGUMENT;
+    if (type == LCU_F32)
+        return delta_rule_t<float>((const float *)proj, row_stride, off_r, off_k, off_v, off_g, off_a, off_l, w2, w0, a_bias, weight, prep, o, state, (float *)out, q_start, ctx_len, state_slot, n, n_req, heads, dk, dv, rank, eps, stream);
+    if (type == LCU_BF16)
+        return delta_rule_t<bf16_t>((const bf16_t *)proj, row_stride, off_r, off_k, off_v, off_g, off_a, off_l, w2, w0, a_bias, weight, prep, o, state, (bf16_t *)out, q_start, ctx_len, state_slot, n, n_req, heads, dk, dv, rank, eps, stream);
+    return LCU_BAD_ARGUMENT;
+}

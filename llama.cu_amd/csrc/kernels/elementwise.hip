@@ -4,11 +4,11 @@
 #include "common.h"
 
 // ---------------------------------------------------------------- embedding gather
-// out[i, :] = table[ids[i], :].  An id outside the table writes NaN into the row
+// out[i, :] = table[ids[i], :] * scale (the product in 32-bit).  An id outside the table writes NaN into the row
 // (the host checks ids before; this keeps a bad id from reading out of bounds).
 template <class TT, class TO>
 __global__ void embedding_gather_kernel(TO *__restrict__ out, const TT *__restrict__ table,
-                                        const int *__restrict__ ids, int d, int vocab) {
+                                        const int *__restrict__ ids, int d, int vocab, float scale) {
     const int row = blockIdx.x;
     const int id = ids[row];
     TO *o = out + (size_t)row * d;
@@ -25,20 +25,20 @@ __global__ void embedding_gather_kernel(TO *__restrict__ out, const TT *__restri
             const In8 in = *(const In8 *)(t + c);
             Out8 res;
 #pragma unroll
-            for (int e = 0; e < 8; ++e) res.v[e] = from_f32<TO>(to_f32(in.v[e]));
+            for (int e = 0; e < 8; ++e) res.v[e] = from_f32<TO>(to_f32(in.v[e]) * scale);
             *(Out8 *)(o + c) = res;
         }
         return;
     }
-    for (int c = threadIdx.x; c < d; c += blockDim.x) o[c] = from_f32<TO>(to_f32(t[c]));
+    for (int c = threadIdx.x; c < d; c += blockDim.x) o[c] = from_f32<TO>(to_f32(t[c]) * scale);
 }
 
 LCU_API int lcu_embedding_gather(void *out, int out_type, const void *table, int table_type,
-                                 const int *ids, int n, int d, int vocab, hipStream_t stream) {
+                                 const int *ids, int n, int d, int vocab, float scale, hipStream_t stream) {
     if (n <= 0) return LCU_OK;
     if (d <= 0 || vocab <= 0) return LCU_BAD_ARGUMENT;
     dim3 grid(n), block(256);
-#define GO(TT, TO) embedding_gather_kernel<TT, TO><<<grid, block, 0, stream>>>((TO *)out, (const TT *)table, ids, d, vocab)
+#define GO(TT, TO) embedding_gather_kernel<TT, TO><<<grid, block, 0, stream>>>((TO *)out, (const TT *)table, ids, d, vocab, scale)
     if (table_type == LCU_F32 && out_type == LCU_F32) GO(float, float);
     else if (table_type == LCU_BF16 && out_type == LCU_F32) GO(bf16_t, float);
     else if (table_type == LCU_BF16 && out_type == LCU_BF16) GO(bf16_t, bf16_t);

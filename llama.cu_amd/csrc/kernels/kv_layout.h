@@ -9,6 +9,8 @@
 //   values: [kv_head][dim][token in page]               the tokens of one dim are
 //           contiguous: a lane that owns a dim reads a run of tokens.
 // head_dim is a multiple of 8 (the engine asks for 16), page_size a multiple of 8.
+// The values' head size may differ from the keys' (v_dim; any size): the functions that
+// take it describe such a page, those without it the page whose two sizes are equal.
 #pragma once
 #include <stddef.h>
 
@@ -20,4 +22,11 @@ __host__ __device__ inline size_t kv_key_offset(int kv_head, int tok, int dim, i
 }
 __host__ __device__ inline size_t kv_value_offset(int kv_heads, int kv_head, int tok, int dim, int head_dim, int page) {
     return (size_t)kv_heads * head_dim * page + ((size_t)kv_head * head_dim + dim) * page + tok;
+}
+
+__host__ __device__ inline size_t kv_page_elems(int kv_heads, int head_dim, int v_dim, int page) {
+    return (size_t)kv_heads * (head_dim + v_dim) * page;
+}
+__host__ __device__ inline size_t kv_value_offset(int kv_heads, int kv_head, int tok, int dim, int head_dim, int v_dim, int page) {
+    return (size_t)kv_heads * head_dim * page + ((size_t)kv_head * v_dim + dim) * page + tok;
 }

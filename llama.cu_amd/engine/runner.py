@@ -140,13 +140,16 @@ class ModelRunner:
         self.groups = [CacheGroup((tokens + ps - 1) // ps, ps, p[0], slack=1 if p[0] else 0) for p, ps in zip(pools, page_of)]
         # whether every need's state of fixed size can be cut back to a shorter length (the manager knows what its
         # pages and windows can); a request that cannot be cut back gives up what cannot and is computed again
-        self.can_truncate = all(n.can_truncate for n in needs if n is not None)
+        own_states = self.model.own_states()
+        self.can_truncate = all(n.can_truncate for n in needs if n is not None) \
+            and all(s.can_truncate for states in own_states for s in states.values())
         self.cache = CacheManager(self.groups, self.max_seqs, can_truncate=self.can_truncate)
         self.caches: List[LayerCache] = []
         for i, (entry, need) in enumerate(zip(spec.run_order, needs)):
             if entry.cache_of is not None:
                 src = self.caches[entry.cache_of]
-                self.caches.append(LayerCache(group=src.group, pages=src.pages, writes=False, state=src.state))
+                self.caches.append(LayerCache(group=src.group, pages=src.pages, writes=False, state=src.state,
+                                              page_size=src.page_size))
             elif need is None:
                 self.caches.append(LayerCache())
             else:
@@ -160,6 +163,8 @@ class ModelRunner:
                     torch.cuda.empty_cache()
                     made = need.allocate(group, pages, ps, self.max_seqs, self.dtype, self.device)
                 self.caches.append(made)
+        for made, states in zip(self.caches, own_states):       # what each entry's block keeps itself, per request
+            made.more = {name: s.allocate(-1, 0, 0, self.max_seqs, self.dtype, self.device).state for name, s in states.items()}
         max_pages = [(self.max_model_len + g.page_size - 1) // g.page_size for g in self.groups]
         self.builder = BatchBuilder(self.cache, self.max_batch_tokens, self.max_seqs, max_pages, self.device)
         # a debugging aid: pages that were given back, or went to another request, since the last step are
@@ -185,9 +190,9 @@ class ModelRunner:
         engine's memory is asked of the driver in one allocation (reserve_in_one_piece)."""
         from .. import models  # noqa: F401  (registers the architectures)
         device = require_gpu(device)
-        arch, cfg = load_config(folder)
-        spec = arch.build_spec(cfg)
         files = open_safetensors(folder)
+        arch, cfg = load_config(folder, shapes={n: tuple(f.shape(n)) for f in files for n in f.names()})
+        spec = arch.build_spec(cfg)
         model = DecoderModel(spec)
         if one_piece:
             reserve_in_one_piece(device, engine_bytes(spec, model.tensors(), DTYPES[dtype], device, int(kw.get("page_size", 16)),

@@ -21,7 +21,7 @@ import torch
 from .runner import ModelRunner
 
 PAGE_SIZE = 16            # the default: divides 64, so a request's pages never exceed its count rounded up to 64
-MAX_LIVE = 8              # the default number of state slots (a trace holds up to four live requests)
+MAX_LIVE = 4              # the default number of state slots: a trace holds up to four live requests, so slots change hands
 
 
 class TraceReplayer:

@@ -8,7 +8,7 @@ CPU path: a tensor that is not on the GPU is an error.
 from __future__ import annotations
 
 import ctypes
-from typing import Optional
+from typing import Dict, Optional
 
 import torch
 
@@ -132,8 +132,8 @@ def _check(rc: int, name: str) -> None:
 # ------------------------------------------------------------------ elementwise
 
 
-def embedding_gather(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
-    """``out[i, :] = table[ids[i], :]`` (converted to ``out``'s type)."""
+def embedding_gather(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor, scale: float = 1.0) -> torch.Tensor:
+    """``out[i, :] = table[ids[i], :] * scale`` (the product in 32-bit, converted to ``out``'s type)."""
     _gpu(table, ids, out)
     _rows(table, "embedding table"); _contig(table, "embedding table"); _contig(out, "embedding out")
     n = ids.numel()
@@ -142,7 +142,7 @@ def embedding_gather(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor) 
         raise KernelError(f"embedding out: shape {tuple(out.shape)}, expected {(n, table.shape[1])}")
     lib = build.load("elementwise")
     _check(lib.lcu_embedding_gather(_ptr(out), _type(out, "embedding out"), _ptr(table), _type(table, "embedding table"),
-                                    _ptr(ids), n, table.shape[1], table.shape[0], _stream()), "embedding_gather")
+                                    _ptr(ids), n, table.shape[1], table.shape[0], ctypes.c_float(scale), _stream()), "embedding_gather")
     return out
 
 
@@ -290,14 +290,15 @@ def rope_kv_store(qkv: torch.Tensor, positions: torch.Tensor, n_heads: int, n_kv
 
 
 def _attention_args(q, out, cache, block_table, q_start, ctx_len, req_of_token, n_heads, n_kv_heads, head_dim,
-                    page_size):
+                    page_size, value_dim: int = 0):
     _gpu(q, out, cache, block_table, q_start, ctx_len, req_of_token)
     _rows(q, "attention q"); _rows(out, "attention out")
     n = q.shape[0]
-    if q.shape[1] < n_heads * head_dim or out.shape != (n, n_heads * head_dim) or out.dtype != q.dtype:
+    value_dim = value_dim or head_dim
+    if q.shape[1] < n_heads * head_dim or out.shape != (n, n_heads * value_dim) or out.dtype != q.dtype:
         raise KernelError("attention: q or out has a wrong shape or type")
-    if cache.dtype != q.dtype or not cache.is_contiguous() or cache.dim() != 3 or cache.shape[1] != 2 \
-            or cache.shape[2] != n_kv_heads * head_dim * page_size:
+    if cache.dtype != q.dtype or not cache.is_contiguous() or cache.dim() != 3 \
+            or cache.shape[1] * cache.shape[2] != n_kv_heads * (head_dim + value_dim) * page_size:
         raise KernelError("attention: cache has a wrong shape, type or layout")
     if block_table.dim() != 2 or block_table.dtype != torch.int32 or not block_table.is_contiguous():
         raise KernelError("attention: block_table must be a contiguous int32 [requests, pages]")
@@ -311,13 +312,15 @@ def _attention_args(q, out, cache, block_table, q_start, ctx_len, req_of_token, 
 def paged_attention_generic(q: torch.Tensor, out: torch.Tensor, cache: torch.Tensor, block_table: torch.Tensor,
                             q_start: torch.Tensor, ctx_len: torch.Tensor, req_of_token: torch.Tensor,
                             n_heads: int, n_kv_heads: int, head_dim: int, page_size: int, scale: float,
-                            window: int = 0, head_slopes: Optional[torch.Tensor] = None) -> torch.Tensor:
+                            window: int = 0, head_slopes: Optional[torch.Tensor] = None, value_dim: int = 0) -> torch.Tensor:
     """Causal attention of the step's queries over the paged cache (every shape).  ``head_slopes``
-    (float32 [n_heads]) adds ``slope[h] * (key position - query position)`` to the scaled scores."""
+    (float32 [n_heads]) adds ``slope[h] * (key position - query position)`` to the scaled scores.
+    ``value_dim``: the values' head size if it is not the keys' (``out`` is ``[n, n_heads * value_dim]``)."""
     n = _attention_args(q, out, cache, block_table, q_start, ctx_len, req_of_token, n_heads, n_kv_heads, head_dim,
-                        page_size)
-    if head_dim % 8 or head_dim > 256:
-        raise KernelError(f"attention: head_dim {head_dim} must be a multiple of 8, at most 256")
+                        page_size, value_dim)
+    value_dim = value_dim or head_dim
+    if head_dim % 8 or head_dim > 256 or value_dim > 256:
+        raise KernelError(f"attention: head_dim {head_dim} must be a multiple of 8, and it and the values' {value_dim} at most 256")
     if head_slopes is not None:
         _gpu(head_slopes)
         if head_slopes.dtype != torch.float32 or head_slopes.shape != (n_heads,) or not head_slopes.is_contiguous():
@@ -325,7 +328,7 @@ def paged_attention_generic(q: torch.Tensor, out: torch.Tensor, cache: torch.Ten
     lib = build.load("attention_generic")
     _check(lib.lcu_paged_attention_generic(_ptr(q), q.stride(0), _ptr(out), out.stride(0), _type(q, "q"), _ptr(cache),
                                            _ptr(block_table), block_table.shape[1], _ptr(q_start), _ptr(ctx_len),
-                                           _ptr(req_of_token), n, n_heads, n_kv_heads, head_dim, page_size,
+                                           _ptr(req_of_token), n, n_heads, n_kv_heads, head_dim, value_dim, page_size,
                                            ctypes.c_float(scale), int(window), _ptr(head_slopes), _stream()), "paged_attention_generic")
     return out
 
@@ -545,14 +548,15 @@ def decode_splits(n_req: int, n_heads: int, n_kv_heads: int, max_ctx_len: int) -
 
 def paged_attention(q: torch.Tensor, out: torch.Tensor, cache: torch.Tensor, step, group: int, n_heads: int,
                     n_kv_heads: int, head_dim: int, page_size: int, scale: float, window: int = 0,
-                    force_generic: bool = False, head_slopes: Optional[torch.Tensor] = None) -> torch.Tensor:
+                    force_generic: bool = False, head_slopes: Optional[torch.Tensor] = None, value_dim: int = 0) -> torch.Tensor:
     """Attention for the batch ``step`` (an engine.batch.StepContext) over cache group
     ``group``: picks the kernel for the batch's shape and type.  A bias inside the scores
     (``head_slopes``) is the generic kernel's: the matrix-core kernels take none."""
     bt = step.block_table(group)
-    if force_generic or head_slopes is not None or not mfma_attention_supported(q, n_heads, n_kv_heads, head_dim, page_size):
+    if force_generic or head_slopes is not None or (value_dim and value_dim != head_dim) \
+            or not mfma_attention_supported(q, n_heads, n_kv_heads, head_dim, page_size):
         return paged_attention_generic(q, out, cache, bt, step.q_start, step.ctx_len, step.req_of_token, n_heads,
-                                       n_kv_heads, head_dim, page_size, scale, window, head_slopes)
+                                       n_kv_heads, head_dim, page_size, scale, window, head_slopes, value_dim)
     n = _attention_args(q, out, cache, bt, step.q_start, step.ctx_len, step.req_of_token, n_heads, n_kv_heads, head_dim,
                         page_size)
     if step.decode_only:
@@ -948,4 +952,202 @@ def gemm_skinny_f32(x: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor
     lib = build.load("gemm_skinny")
     _check(lib.lcu_gemm_skinny_f32(_ptr(x), x.stride(0), _ptr(w), w.stride(0), _ptr(out), out.stride(0), m, n, k,
                                    int(bool(accumulate)), _stream()), "gemm_skinny_f32")
+    return out
+
+
+# ------------------------------------------------------------------ layer norm, short convolution
+
+
+def _f32_vec(t: Optional[torch.Tensor], what: str, size: int) -> None:
+    if t is not None and (t.dtype != torch.float32 or t.shape != (size,) or not t.is_contiguous()):
+        raise KernelError(f"{what}: must be contiguous float32 [{size}], got {t.dtype} {tuple(t.shape)}")
+
+
+def layernorm(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, eps: float, out: torch.Tensor,
+              delta: Optional[torch.Tensor] = None, weight2: Optional[torch.Tensor] = None,
+              bias2: Optional[torch.Tensor] = None, out2: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``y = (x' - mean) * rsqrt(var + eps) * weight + bias`` with ``x' = x + delta`` (rows, or planes
+    ``[planes, n, d]`` that are added one after the other), in 32-bit; ``x`` (float32, the residual stream) takes
+    the sum in.  With ``weight2``, ``bias2``, ``out2`` a second norm of the same rows is written in the same pass."""
+    _gpu(x, weight, bias, out, delta, weight2, bias2, out2)
+    _rows(x, "norm input"); _contig(x, "norm input"); _contig(out, "norm out")
+    n, d = x.shape
+    if x.dtype != torch.float32:
+        raise KernelError("layernorm: the input (the residual stream) must be float32")
+    _f32_vec(weight, "layernorm weight", d); _f32_vec(bias, "layernorm bias", d)
+    _f32_vec(weight2, "layernorm weight", d); _f32_vec(bias2, "layernorm bias", d)
+    if out.shape != (n, d) or (out2 is not None and (out2.shape != (n, d) or out2.dtype != out.dtype or not out2.is_contiguous())):
+        raise KernelError("layernorm out: wrong shape, type or layout")
+    if (weight2 is None) != (out2 is None) or (weight2 is None) != (bias2 is None):
+        raise KernelError("layernorm: a second norm needs its weight, its bias and its output")
+    planes = 0
+    if delta is not None:
+        _contig(delta, "norm delta")
+        if delta.shape[-2:] != (n, d) or delta.dim() not in (2, 3):
+            raise KernelError(f"norm delta: shape {tuple(delta.shape)}, expected [{n}, {d}] or planes of it")
+        planes = delta.shape[0] if delta.dim() == 3 else 1
+    lib = build.load("norm_conv")
+    _check(lib.lcu_layernorm(_ptr(x), _ptr(delta), _type(delta, "norm delta") if delta is not None else -1, planes,
+                             _ptr(weight), _ptr(bias), _ptr(out), _ptr(weight2), _ptr(bias2), _ptr(out2),
+                             _type(out, "norm out"), n, d, ctypes.c_float(eps), _stream()), "layernorm")
+    return out
+
+
+def short_conv(h: torch.Tensor, weight: torch.Tensor, state: torch.Tensor, out: torch.Tensor, step, update: bool = True) -> torch.Tensor:
+    """``out = h + conv(h)``, a causal convolution over each request's rows on every channel, ``sets`` of them at
+    once: ``h [sets, n, d]``, ``weight [sets, d, taps]``, ``state [slots, sets, taps - 1, d]`` (float32: the last
+    ``taps - 1`` rows that each request has fed so far), ``out [sets, n, d]``.  ``conv(h)[t] = sum_j weight[:, j] *
+    h[t - taps + 1 + j]``; rows before a request's first are zeros.  ``update``: the states then take this step's
+    rows in.  ``step``: the batch (``q_start``, ``ctx_len``, ``req_of_token``, ``state_slot``)."""
+    _gpu(h, weight, state, out)
+    _contig(h, "conv input"); _contig(weight, "conv weight"); _contig(state, "conv state"); _contig(out, "conv out")
+    if h.dim() != 3 or out.shape != h.shape or weight.dim() != 3 or weight.shape[:2] != (h.shape[0], h.shape[2]):
+        raise KernelError(f"short_conv: h {tuple(h.shape)}, weight {tuple(weight.shape)}, out {tuple(out.shape)} do not fit")
+    sets, n, d = h.shape
+    taps = weight.shape[2]
+    if state.dtype != torch.float32 or state.dim() != 4 or state.shape[1:] != (sets, taps - 1, d):
+        raise KernelError(f"short_conv: state must be float32 [slots, {sets}, {taps - 1}, {d}], got {state.dtype} {tuple(state.shape)}")
+    if n != step.n or max(step.state_slots, default=0) >= state.shape[0]:
+        raise KernelError("short_conv: the rows are not the step's, or a request's slot lies outside the state")
+    lib = build.load("norm_conv")
+    _check(lib.lcu_short_conv(_ptr(h), _type(h, "conv input"), ctypes.c_longlong(n * d), _ptr(weight), _type(weight, "conv weight"),
+                              _ptr(state), _ptr(out), _type(out, "conv out"), ctypes.c_longlong(n * d), _ptr(step.q_start),
+                              _ptr(step.ctx_len), _ptr(step.req_of_token), _ptr(step.state_slot), n, step.n_req, d, taps, sets,
+                              int(bool(update)), _stream()), "short_conv")
+    return out
+
+
+# ------------------------------------------------------------------ norm of whole projections, cache write
+
+
+def qk_norm_store(qkv: torch.Tensor, positions: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: int, value_dim: int,
+                  q_weight: Optional[torch.Tensor], k_weight: Optional[torch.Tensor], eps: float, temp_coef: float,
+                  temp_every: int, cache: Optional[torch.Tensor], slots: Optional[torch.Tensor], page_size: int) -> None:
+    """For attention without a rotation: the queries of ``qkv [n, heads * head_dim (+ kv_heads * (head_dim +
+    value_dim))]`` are divided by the root mean square over the whole projection and multiplied by ``q_weight``
+    (None: no norm) and by ``1 + temp_coef * ln(floor((p + 1) / temp_every) + 1)`` at position ``p`` (0: no such
+    factor), in place; the keys likewise (``k_weight``) on their way into ``cache`` at ``slots``, the values as they
+    are.  ``cache=None``: the rows hold queries only."""
+    _gpu(qkv, positions, q_weight, k_weight, cache, slots)
+    _rows(qkv, "qkv")
+    n = qkv.shape[0]
+    store = cache is not None
+    need = n_heads * head_dim + (n_kv_heads * (head_dim + value_dim) if store else 0)
+    if qkv.shape[1] != need or qkv.stride(1) != 1:
+        raise KernelError(f"qkv: width {qkv.shape[1]}, expected {need}")
+    _i32(positions, "positions", n)
+    _f32_vec(q_weight, "query norm weight", n_heads * head_dim)
+    _f32_vec(k_weight, "key norm weight", n_kv_heads * head_dim)
+    if head_dim % 8:
+        raise KernelError(f"head_dim {head_dim} must be a multiple of 8")
+    if store:
+        _i32(slots, "cache slots", n)
+        _contig(cache, "cache")
+        if cache.dtype != qkv.dtype or cache.dim() != 3 or cache.shape[1] * cache.shape[2] != n_kv_heads * (head_dim + value_dim) * page_size:
+            raise KernelError(f"cache: {cache.dtype} {tuple(cache.shape)} does not hold pages of {n_kv_heads} x ({head_dim} + {value_dim}) x {page_size} {qkv.dtype}")
+    lib = build.load("qk_norm")
+    _check(lib.lcu_qk_norm_store(_ptr(qkv), _type(qkv, "qkv"), n, qkv.stride(0), _ptr(positions), _ptr(slots), _ptr(q_weight),
+                                 _ptr(k_weight), _ptr(cache), n_heads, n_kv_heads, head_dim, value_dim, page_size,
+                                 ctypes.c_float(eps), ctypes.c_float(temp_coef), int(temp_every or 1), int(store), _stream()),
+           "qk_norm_store")
+
+
+# ------------------------------------------------------------------ the generalised delta rule
+
+
+def delta_rule(proj: torch.Tensor, offsets: Dict[str, int], w2: torch.Tensor, w0: torch.Tensor, a_bias: torch.Tensor,
+               weight: torch.Tensor, state: torch.Tensor, step, heads: int, key_dim: int, value_dim: int, eps: float,
+               out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """The recurrent mixer ``S <- diag(w) S - (a u)(u^T S) + k v^T``, ``o = S^T r`` over the step's rows, request by
+    request from each request's state (``state [slots, heads, key_dim, value_dim]`` float32, taken as zero at a
+    request's position 0 and left as the step's last token makes it).  ``proj [n, *]`` holds the projections at the
+    columns ``offsets``: ``r, k, v, g, a`` (heads * dim each) and ``l`` (the low-rank projection whose ``tanh``,
+    times ``w2 [heads * key_dim, rank]`` plus ``w0``, gives the decay ``w = exp(-exp(-1/2) sigmoid(.))``); ``a =
+    sigmoid(a_lin + a_bias)``, ``u = k / sqrt(sum k^2 + 1e-6)``.  Returns ``o`` of each head divided by its root mean
+    square (``eps``), times ``weight``, times ``sigmoid(g)``, in ``proj``'s type ``[n, heads * value_dim]``."""
+    _gpu(proj, w2, w0, a_bias, weight, state, out)
+    _rows(proj, "delta projections")
+    n = proj.shape[0]
+    hk, hv = heads * key_dim, heads * value_dim
+    if w2.dim() != 2 or w2.shape[0] != hk or w2.dtype != torch.float32 or not w2.is_contiguous():
+        raise KernelError(f"delta_rule: w2 must be contiguous float32 [{hk}, rank], got {w2.dtype} {tuple(w2.shape)}")
+    rank = w2.shape[1]
+    _f32_vec(w0, "delta_rule w0", hk); _f32_vec(a_bias, "delta_rule a_bias", hk); _f32_vec(weight, "delta_rule weight", hv)
+    widths = {"r": hk, "k": hk, "v": hv, "g": hv, "a": hk, "l": rank}
+    for name, width in widths.items():
+        if name not in offsets or offsets[name] < 0 or offsets[name] + width > proj.shape[1]:
+            raise KernelError(f"delta_rule: the columns of {name!r} lie outside the projections' {proj.shape[1]} columns")
+    if proj.stride(1) != 1:
+        raise KernelError("delta_rule: the projections' columns must be contiguous")
+    if state.dtype != torch.float32 or not state.is_contiguous() or state.dim() != 4 or state.shape[1:] != (heads, key_dim, value_dim):
+        raise KernelError(f"delta_rule: state must be contiguous float32 [slots, {heads}, {key_dim}, {value_dim}]")
+    if n != step.n or max(step.state_slots, default=0) >= state.shape[0]:
+        raise KernelError("delta_rule: the rows are not the step's, or a request's slot lies outside the state")
+    if out is None:
+        out = torch.empty((n, hv), dtype=proj.dtype, device=proj.device)
+    if out.shape != (n, hv) or out.dtype != proj.dtype or not out.is_contiguous():
+        raise KernelError("delta_rule out: wrong shape, type or layout")
+    prep = torch.empty((n, heads, 5, key_dim), dtype=torch.float32, device=proj.device)
+    o = torch.empty((n, hv), dtype=torch.float32, device=proj.device)
+    lib = build.load("delta_rule")
+    _check(lib.lcu_delta_rule(_ptr(proj), _type(proj, "delta projections"), proj.stride(0), offsets["r"], offsets["k"], offsets["v"],
+                              offsets["g"], offsets["a"], offsets["l"], _ptr(w2), _ptr(w0), _ptr(a_bias), _ptr(weight), _ptr(prep),
+                              _ptr(o), _ptr(state), _ptr(out), _ptr(step.q_start), _ptr(step.ctx_len), _ptr(step.state_slot), n,
+                              step.n_req, heads, key_dim, value_dim, rank, ctypes.c_float(eps), _stream()), "delta_rule")
+    return out
+
+
+# ------------------------------------------------------------------ mixture of experts
+
+
+def moe_route(h: torch.Tensor, router: torch.Tensor, top: int):
+    """``(ids, weights)``, each ``[n, top]``: every row's ``top`` experts by ``router @ h`` (32-bit; ties go to the
+    lower index), largest first, with the weight ``sigmoid`` of that logit."""
+    _gpu(h, router)
+    _rows(h, "moe input"); _contig(h, "moe input"); _contig(router, "router")
+    n, d = h.shape
+    if router.dtype != torch.float32 or router.dim() != 2 or router.shape[1] != d:
+        raise KernelError(f"moe_route: the router must be float32 [experts, {d}], got {router.dtype} {tuple(router.shape)}")
+    experts = router.shape[0]
+    if not 0 < top <= experts or experts > 1024:
+        raise KernelError(f"moe_route: top {top} of {experts} experts is not supported (at most 1024 experts)")
+    ids = torch.empty((n, top), dtype=torch.int32, device=h.device)
+    wts = torch.empty((n, top), dtype=torch.float32, device=h.device)
+    lib = build.load("moe")
+    _check(lib.lcu_moe_route(_ptr(h), _type(h, "moe input"), _ptr(router), _ptr(ids), _ptr(wts), n, d, experts, top, _stream()),
+           "moe_route")
+    return ids, wts
+
+
+def moe_experts(h: torch.Tensor, ids: torch.Tensor, wts: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor,
+                out: torch.Tensor) -> torch.Tensor:
+    """``out[t] += sum over t's experts e of  w_down[e] @ gelu(w_up[e] @ (weight * h[t]))`` (the exact gelu; the
+    weight multiplies the expert's input).  ``w_up [experts, ff, d]``, ``w_down [experts, d, ff]`` in ``h``'s type,
+    ``out`` float32 ``[n, d]``."""
+    _gpu(h, ids, wts, w_up, w_down, out)
+    _rows(h, "moe input")
+    for t, what in ((h, "moe input"), (ids, "moe ids"), (wts, "moe weights"), (w_up, "moe up"), (w_down, "moe down"), (out, "moe out")):
+        _contig(t, what)
+    n, d = h.shape
+    if w_up.dim() != 3 or w_down.dim() != 3 or w_up.shape[2] != d or w_down.shape != (w_up.shape[0], d, w_up.shape[1]) \
+            or w_up.dtype != h.dtype or w_down.dtype != h.dtype:
+        raise KernelError(f"moe_experts: up {tuple(w_up.shape)} {w_up.dtype} and down {tuple(w_down.shape)} {w_down.dtype} do not fit rows of {d} {h.dtype}")
+    experts, ff = w_up.shape[0], w_up.shape[1]
+    top = ids.shape[1] if ids.dim() == 2 else 0
+    if ids.shape != (n, top) or ids.dtype != torch.int32 or wts.shape != (n, top) or wts.dtype != torch.float32 or top < 1:
+        raise KernelError("moe_experts: ids (int32) and weights (float32) must be [n, top]")
+    if out.shape != (n, d) or out.dtype != torch.float32:
+        raise KernelError("moe_experts: out must be float32 [n, d]")
+    per = 8 if h.dtype == torch.bfloat16 else 4
+    if d % per or ff % per:
+        raise KernelError(f"moe_experts: the width {d} and the experts' {ff} must be multiples of {per}")
+    lib = build.load("moe")
+    tile = lib.lcu_moe_tile_rows()
+    total = n * top
+    max_tiles = min(total, total // tile + experts)
+    ints = torch.empty(total + 3 * max_tiles + 1, dtype=torch.int32, device=h.device)
+    act = torch.empty((total, ff), dtype=h.dtype, device=h.device)
+    y = torch.empty((total, d), dtype=torch.float32, device=h.device) if top > 1 else None
+    _check(lib.lcu_moe_experts(_ptr(h), _type(h, "moe input"), _ptr(ids), _ptr(wts), _ptr(ints), max_tiles, _ptr(w_up),
+                               _ptr(w_down), _ptr(act), _ptr(y), _ptr(out), n, d, ff, experts, top, _stream()), "moe_experts")
     return out

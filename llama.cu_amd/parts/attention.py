@@ -22,8 +22,18 @@ from ..weights.loader import fused_rows
 
 class Attention(Part):
 
+    # the tensors' names under the part's own, as files with config.json's names hold them; ``names`` replaces any
+    NAMES = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight",
+             "q_norm": "q_norm.weight", "k_norm": "k_norm.weight"}
+
     def __init__(self, hidden_size: int, heads: int, kv_heads: int, head_dim: int, scale: Optional[float] = None,
-                 window: int = 0, position: Optional[PartSpec] = None, shares_kv: bool = False, page_size: int = 0):
+                 window: int = 0, position: Optional[PartSpec] = None, shares_kv: bool = False, page_size: int = 0,
+                 value_dim: int = 0, projection_norm_eps: Optional[float] = None, query_temperature=None,
+                 names: Optional[Dict[str, str]] = None):
+        """``value_dim``: the values' head size if it is not ``head_dim``.  ``projection_norm_eps``: queries and keys
+        are divided by the root mean square over their whole projection (all heads at once) and multiplied by a
+        weight per column (tensors ``q_norm``, ``k_norm``).  ``query_temperature = (coef, every)``: the query at
+        position ``p`` is multiplied by ``1 + coef * ln(floor((p + 1) / every) + 1)``."""
         if heads % kv_heads:
             raise ValueError(f"attention: {heads} heads are no multiple of {kv_heads} key/value heads")
         if head_dim % 16 or head_dim > 256:
@@ -32,6 +42,18 @@ class Attention(Part):
         self.hidden_size, self.heads, self.kv_heads, self.head_dim = int(hidden_size), int(heads), int(kv_heads), int(head_dim)
         self.scale = float(scale) if scale is not None else float(head_dim) ** -0.5
         self.window = int(window or 0)
+        self.value_dim = int(value_dim or head_dim)
+        if self.value_dim > 256:
+            raise ValueError(f"attention: value_dim {value_dim} is not supported by the kernels (at most 256)")
+        self.norm_eps = None if projection_norm_eps is None else float(projection_norm_eps)
+        self.q_temp = None
+        if query_temperature is not None:
+            coef, every = query_temperature
+            if int(every) < 1:
+                raise ValueError(f"attention: the query temperature's step {every} must be at least 1")
+            self.q_temp = (float(coef), int(every))
+        self.names = dict(self.NAMES, **(names or {}))
+        self.q_norm = self.k_norm = None
         self.own_page_size = int(page_size or 0)  # tokens per page of this layer's cache; 0: the engine's default
         self.shares_kv = bool(shares_kv)          # reads another layer's keys and values: has q and o only
         self.position = make_part("position", position or PartSpec("none"))
@@ -40,18 +62,23 @@ class Attention(Part):
         self.page_size = 0
 
     def tensors(self) -> Dict[str, TensorSpec]:
-        d, nh, nkv, dh = self.hidden_size, self.heads, self.kv_heads, self.head_dim
-        t = {"q_proj.weight": TensorSpec((nh * dh, d)), "o_proj.weight": TensorSpec((d, nh * dh))}
+        d, nh, nkv, dh, dv, nm = self.hidden_size, self.heads, self.kv_heads, self.head_dim, self.value_dim, self.names
+        t = {nm["q"]: TensorSpec((nh * dh, d)), nm["o"]: TensorSpec((d, nh * dv))}
         if not self.shares_kv:
-            t["k_proj.weight"] = TensorSpec((nkv * dh, d))
-            t["v_proj.weight"] = TensorSpec((nkv * dh, d))
+            t[nm["k"]] = TensorSpec((nkv * dh, d))
+            t[nm["v"]] = TensorSpec((nkv * dv, d))
+        if self.norm_eps is not None:
+            t[nm["q_norm"]] = TensorSpec((nh * dh,), init="one_plus_normal")
+            if not self.shares_kv:
+                t[nm["k_norm"]] = TensorSpec((nkv * dh,), init="one_plus_normal")
         return t
 
     def fused_groups(self, dtype, device):
-        return [] if self.shares_kv else [(("q_proj.weight", "k_proj.weight", "v_proj.weight"), 0)]
+        return [] if self.shares_kv else [((self.names["q"], self.names["k"], self.names["v"]), 0)]
 
     def cache_need(self):
-        return PagedKV(self.kv_heads, self.head_dim, self.window, self.own_page_size)
+        return PagedKV(self.kv_heads, self.head_dim, self.window, self.own_page_size,
+                       self.value_dim if self.value_dim != self.head_dim else 0)
 
     def decode_splits(self, batch: int, max_ctx_len: int) -> int:
         """Into how many parts the decode kernel should cut each request's keys when ``batch``
@@ -59,12 +86,16 @@ class Attention(Part):
         return ops.decode_splits(batch, self.heads, self.kv_heads, max_ctx_len)
 
     def load(self, tensors, build: BuildContext) -> None:
+        nm = self.names
         if self.shares_kv:
-            self.w_qkv = Weight(tensors["q_proj.weight"], build)
+            self.w_qkv = Weight(tensors[nm["q"]], build)
         else:
             # one matrix with the rows of q, then k, then v: in place where the loader laid them out so
-            self.w_qkv = Weight(fused_rows([tensors["q_proj.weight"], tensors["k_proj.weight"], tensors["v_proj.weight"]]), build)
-        self.w_o = Weight(tensors["o_proj.weight"], build)
+            self.w_qkv = Weight(fused_rows([tensors[nm["q"]], tensors[nm["k"]], tensors[nm["v"]]]), build)
+        self.w_o = Weight(tensors[nm["o"]], build)
+        if self.norm_eps is not None:            # the kernel takes the norms' weights in 32-bit
+            self.q_norm = tensors[nm["q_norm"]].float().contiguous()
+            self.k_norm = None if self.shares_kv else tensors[nm["k_norm"]].float().contiguous()
         self.position.load({}, build)
         # a position encoding that is its rotation tables alone (apply() does nothing of its own)
         self._rotation_only = type(self.position).apply is Part.apply
@@ -76,6 +107,8 @@ class Attention(Part):
             why = ops.mfma_attention_refusal(self.dtype, self.heads, self.kv_heads, self.head_dim, self.own_page_size or self.page_size)
             if why is None and self.position.score_slopes() is not None:
                 why = "the position encoding is a bias inside the scores, which the matrix-core kernels do not take"
+            if why is None and self.value_dim != self.head_dim:
+                why = f"the values' head size {self.value_dim} is not the keys' {self.head_dim}"
             if why is not None:
                 ops.say_once(f"attention with {self.heads} heads of {self.head_dim} in {self.kv_heads} groups runs on the generic "
                              f"kernel, not on the matrix cores: {why}")
@@ -85,7 +118,7 @@ class Attention(Part):
         the host, and go to the device with the step's arrays; ``forward`` then launches work whose sizes follow from
         the step's sizes alone."""
         page_size = self.own_page_size or self.page_size
-        if self.dtype == torch.bfloat16 and self.position.score_slopes() is None \
+        if self.dtype == torch.bfloat16 and self.position.score_slopes() is None and self.value_dim == self.head_dim \
                 and ops.mfma_attention_refusal(self.dtype, self.heads, self.kv_heads, self.head_dim, page_size) is None:
             ops.plan_attention(step, self.heads, self.kv_heads, self.window)
 
@@ -101,8 +134,15 @@ class Attention(Part):
         product anyway."""
         return self.dtype == torch.bfloat16 and n_rows <= ops.ADD_NORM_MAX_ROWS and skinny_takes(n_rows, self.w_qkv, preferred=True)
 
-    def forward(self, h, step, cache, into=None, planes_ok=False):
-        nh, nkv, dh = self.heads, self.kv_heads, self.head_dim
+    def forward(self, h, step, cache, into=None, planes_ok=False, out_dtype=None):
+        """``out_dtype``: the type of the branch's output if it is not the compute type (a block that adds
+        several branches before the residual sum asks for float32)."""
+        nh, nkv, dh, dv = self.heads, self.kv_heads, self.head_dim, self.value_dim
+        plain = self.norm_eps is None and self.q_temp is None       # nothing but a rotation between the product and the cache
+        if not plain and self.position.rotary_tables() is not None:
+            raise ops.KernelError("attention: a norm over the whole projection or a query temperature together with a rotation is not supported")
+        if plain and dv != dh:
+            raise ops.KernelError("attention: values of another head size than the keys' need the path without a rotation")
         if self.shares_kv == cache.writes:
             raise ops.KernelError("attention: a layer that shares another's keys and values must be given that "
                                   "layer's cache in the run order (and only such a layer)")
@@ -112,7 +152,7 @@ class Attention(Part):
         store = cache.writes and not self.shares_kv
         n_rows = (h.rows if isinstance(h, ScaledRows) else h).shape[0]
         qkv = None
-        if store and self._rotation_only and rot is not None and pairing == 0 and rot_dim == dh \
+        if plain and store and self._rotation_only and rot is not None and pairing == 0 and rot_dim == dh \
                 and self.dtype == torch.bfloat16 and (skinny_takes(n_rows, self.w_qkv, preferred=True)
                                                       or (not isinstance(h, ScaledRows) and mid_qkv_takes(n_rows, self.w_qkv))):
             # up to 256 rows: the product rotates q and k and writes k and v into the pages itself
@@ -124,12 +164,20 @@ class Attention(Part):
             else:
                 qkv = linear(h, self.w_qkv, out_dtype=self.dtype)
             self.position.apply(qkv, step.positions, nh, 0 if self.shares_kv else nkv, dh)
-            ops.rope_kv_store(qkv, step.positions, nh, nkv, dh, cos, sin, rot_dim, pairing,
-                              cache.pages if store else None, step.slots(cache.group) if store else None,
-                              page_size)
-        out = torch.empty((n_rows, nh * dh), dtype=self.dtype, device=qkv.device)
+            if plain:
+                ops.rope_kv_store(qkv, step.positions, nh, nkv, dh, cos, sin, rot_dim, pairing,
+                                  cache.pages if store else None, step.slots(cache.group) if store else None,
+                                  page_size)
+            else:
+                coef, every = self.q_temp or (0.0, 1)
+                ops.qk_norm_store(qkv, step.positions, nh, nkv, dh, dv, self.q_norm, self.k_norm, self.norm_eps or 0.0,
+                                  coef, every, cache.pages if store else None,
+                                  step.slots(cache.group) if store else None, page_size)
+        out = torch.empty((n_rows, nh * dv), dtype=self.dtype, device=qkv.device)
         ops.paged_attention(qkv, out, cache.pages, step, cache.group, nh, nkv, dh, page_size, self.scale,
-                            self.window, head_slopes=self.position.score_slopes())
+                            self.window, head_slopes=self.position.score_slopes(), value_dim=dv)
+        if out_dtype is not None and out_dtype != self.dtype:
+            return linear(out, self.w_o, out_dtype=out_dtype)
         if into is not None:
             residual, norm = into
             fused = linear_into_norm(out, self.w_o, residual, norm.weight)

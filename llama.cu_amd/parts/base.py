@@ -84,6 +84,7 @@ class LayerCache:
     writes: bool = True
     state: Optional[torch.Tensor] = None
     page_size: int = 0          # tokens per page of ``pages`` (0: no pages)
+    more: Dict[str, torch.Tensor] = field(default_factory=dict)   # the block's own states by name (``Part.own_states``)
 
 
 class CacheNeed:
@@ -116,21 +117,26 @@ class CacheNeed:
 
 @dataclass(frozen=True)
 class PagedKV(CacheNeed):
-    """Keys and values of every token (or of the last ``window`` tokens), in pages."""
+    """Keys and values of every token (or of the last ``window`` tokens), in pages.  ``value_dim``: the values'
+    head size if it is not the keys' (a page then holds all its keys, then all its values, in one row)."""
     kv_heads: int
     head_dim: int
     window: int = 0          # 0: all tokens
     page_size: int = 0       # tokens per page; 0: the engine's default
+    value_dim: int = 0       # 0: head_dim
 
     def pool(self):
         return (self.window, self.page_size)
 
     def page_bytes(self, page_size: int, elem_size: int) -> int:
-        return 2 * self.kv_heads * self.head_dim * page_size * elem_size
+        return self.kv_heads * (self.head_dim + (self.value_dim or self.head_dim)) * page_size * elem_size
 
     def allocate(self, group, num_pages, page_size, slots, dtype, device) -> LayerCache:
-        pages = torch.zeros((num_pages, 2, self.kv_heads * self.head_dim * page_size), dtype=dtype, device=device)
-        return LayerCache(group=group, pages=pages, page_size=page_size)
+        if self.value_dim and self.value_dim != self.head_dim:
+            shape = (num_pages, 1, self.kv_heads * (self.head_dim + self.value_dim) * page_size)
+        else:
+            shape = (num_pages, 2, self.kv_heads * self.head_dim * page_size)
+        return LayerCache(group=group, pages=torch.zeros(shape, dtype=dtype, device=device), page_size=page_size)
 
 
 @dataclass(frozen=True)
@@ -227,6 +233,14 @@ class Part:
 
     def load(self, tensors: Dict[str, torch.Tensor], build: BuildContext) -> None:
         pass
+
+    def own_states(self) -> Dict[str, "SlotState"]:
+        """block: states of fixed size per request that the block itself keeps, beside what its mixer asks for with
+        ``cache_need`` (the last inputs of a convolution over time, say), by name.  Every entry of the run order
+        gets its own, also one that reads another entry's keys and values; ``forward`` finds them in
+        ``cache.more[name]`` as ``[slots, *shape]``.  Like any SlotState they are not cleared when a slot changes
+        hands: their owner starts them anew at a request's position 0."""
+        return {}
 
     def prepare(self, step) -> None:
         """Called once per step for every layer, on the host, before the step's arrays go to the device and

@@ -1,5 +1,8 @@
 """The arrangement of norm, mixer, norm and feed-forward in one layer.
 
+``parallel``: ``x += mixer(norm1(x)) + ffn(norm2(x))``, both branches reading the same ``x``, each
+optionally through a short causal convolution over time (ParallelBlock below).
+
 ``prenorm``: ``x += mixer(norm1(x)); x += ffn(norm2(x))``
 (llama.cu/src/model/mod.rs:100-157, ``TransformerBlk::new(norm, attention, norm, mlp)``;
 the residual is added where the output and down projections end,
@@ -9,11 +12,13 @@ branch's output as ``pending``, and whoever norms next adds it.
 """
 from __future__ import annotations
 
-from typing import Dict
+from typing import Dict, Optional
 
 import torch
 
-from .base import BuildContext, Part, PartSpec, ScaledRows, TensorSpec, make_part, prefixed, register_part
+from ..kernels import ops
+from .base import BuildContext, Part, PartSpec, ScaledRows, SlotState, TensorSpec, make_part, prefixed, register_part
+from .norm import LayerNorm
 
 
 class PreNormBlock(Part):
@@ -104,3 +109,109 @@ class PreNormBlock(Part):
 
 
 register_part("block", "prenorm", PreNormBlock)
+
+
+class ParallelBlock(Part):
+    """``x += mixer(c1(norm1(x))) + ffn(c2(norm2(x)))``: two norms of the same ``x``, one sum.  The feed-forward
+    (with its norm) may be missing.
+
+    ``conv_taps > 0``: what each branch reads, ``h``, is first replaced by ``h + conv(h)``, a causal convolution
+    over time on each channel with a weight ``[width, taps]`` and no bias (``conv_tensors`` names the two):
+    ``conv(h)[t] = sum_j w[:, j] * h[t - taps + 1 + j]``, zeros before the sequence's start.  The last ``taps - 1``
+    inputs of both branches are state of the request (``own_states``), carried from step to step in 32-bit.
+
+    The branches' outputs are float32 and are added to one another before the norm that follows adds them to the
+    residual stream (``pending``)."""
+
+    def __init__(self, hidden_size: int, norm1: PartSpec, mixer: PartSpec, norm2: Optional[PartSpec] = None,
+                 ffn: Optional[PartSpec] = None, conv_taps: int = 0, conv_tensors=("conv1", "conv2")):
+        if (norm2 is None) != (ffn is None):
+            raise ValueError("parallel block: the second norm and the feed-forward come together or not at all")
+        self.hidden_size, self.taps = int(hidden_size), int(conv_taps or 0)
+        if self.taps > 16:
+            raise ValueError(f"parallel block: a convolution of {conv_taps} taps is not supported (at most 16)")
+        self.conv_tensors = tuple(conv_tensors)
+        self.specs = {"norm1": norm1, "mixer": mixer, "norm2": norm2, "ffn": ffn}
+        self.norm1 = make_part("norm", norm1)
+        self.mixer = make_part("mixer", mixer)
+        self.norm2 = make_part("norm", norm2) if norm2 is not None else None
+        self.ffn = make_part("ffn", ffn) if ffn is not None else None
+        self.sets = 2 if self.ffn is not None else 1
+        self.graph_safe = all(p.graph_safe for _, p in self._children())
+        # two layer norms of the same row are one kernel
+        self._pair = isinstance(self.norm1, LayerNorm) and (self.norm2 is None or (isinstance(self.norm2, LayerNorm)
+                                                                                   and self.norm2.eps == self.norm1.eps))
+        self.conv_weight = None
+
+    def _children(self):
+        return [(self.specs[k].name, getattr(self, k)) for k in ("norm1", "mixer", "norm2", "ffn") if getattr(self, k) is not None]
+
+    def tensors(self) -> Dict[str, TensorSpec]:
+        out = {}
+        for name, part in self._children():
+            for k, v in part.tensors().items():
+                out[prefixed(name, k)] = v
+        if self.taps:
+            for name in self.conv_tensors[:self.sets]:
+                out[name] = TensorSpec((self.hidden_size, self.taps))
+        return out
+
+    def load(self, tensors, build: BuildContext) -> None:
+        for name, part in self._children():
+            pre = name + "." if name else ""
+            part.load({k[len(pre):]: v for k, v in tensors.items() if k.startswith(pre)}, build)
+        if self.taps:       # both convolutions' weights side by side, in 32-bit: one kernel runs the two
+            self.conv_weight = torch.stack([tensors[n].float() for n in self.conv_tensors[:self.sets]]).contiguous()
+        self.dtype = build.dtype
+
+    def fused_groups(self, dtype, device):
+        out = []
+        for name, part in self._children():
+            out += [(tuple(prefixed(name, n) for n in names), pad) for names, pad in part.fused_groups(dtype, device)]
+        return out
+
+    def cache_need(self):
+        return self.mixer.cache_need()
+
+    def own_states(self):
+        if self.taps < 2:
+            return {}
+        return {"conv": SlotState((self.sets, self.taps - 1, self.hidden_size), torch.float32)}
+
+    def prepare(self, step) -> None:
+        for _, part in self._children():
+            part.prepare(step)
+
+    def decode_splits(self, batch: int, max_ctx_len: int) -> int:
+        return int(self.mixer.decode_splits(batch, max_ctx_len))
+
+    @property
+    def takes_planes(self) -> bool:
+        return bool(self.norm1.takes_planes)
+
+    def forward(self, x: torch.Tensor, pending, step, cache, next_norm=None, planes_ok=False):
+        n, d = x.shape
+        conv = self.taps > 0
+        # with a convolution behind them the norms write 32-bit rows, which are rounded once, after the convolution
+        mid = torch.float32 if conv else self.dtype
+        h = torch.empty((self.sets, n, d), dtype=mid, device=x.device)
+        if self._pair:
+            two = self.norm2 is not None
+            ops.layernorm(x, self.norm1.weight, self.norm1.bias, self.norm1.eps, h[0], delta=pending,
+                          weight2=self.norm2.weight if two else None, bias2=self.norm2.bias if two else None,
+                          out2=h[1] if two else None)
+        else:
+            first = self.norm1.forward(x, pending)
+            h = torch.stack([first] + ([self.norm2.forward(x, None)] if self.norm2 is not None else []))
+        if conv:
+            if self.taps > 1 and "conv" not in cache.more:
+                raise ops.KernelError("parallel block: the layer was given no state for its convolutions")
+            state = cache.more["conv"] if self.taps > 1 else torch.empty((1, self.sets, 0, d), dtype=torch.float32, device=x.device)
+            h = ops.short_conv(h, self.conv_weight, state, torch.empty((self.sets, n, d), dtype=self.dtype, device=x.device), step)
+        out = self.mixer.forward(h[0], step, cache, out_dtype=torch.float32)
+        if self.ffn is not None:
+            out = self.ffn.forward(h[1], add_to=out)
+        return out
+
+
+register_part("block", "parallel", ParallelBlock)

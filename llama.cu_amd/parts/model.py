@@ -22,20 +22,23 @@ from .linear import Weight, linear, linear_scaled, skinny_takes
 class TokenEmbedding(Part):
     graph_safe = True
 
-    def __init__(self, vocab_size: int, hidden_size: int):
+    def __init__(self, vocab_size: int, hidden_size: int, scale: float = 1.0, tensor: str = "weight"):
+        """``scale``: every row is multiplied by it (in 32-bit) on its way into the residual stream.
+        ``tensor``: the table's name under the part's."""
         self.vocab_size, self.hidden_size = int(vocab_size), int(hidden_size)
+        self.scale, self.tensor = float(scale), str(tensor)
         self.weight = None
 
     def tensors(self):
-        return {"weight": TensorSpec((self.vocab_size, self.hidden_size))}
+        return {self.tensor: TensorSpec((self.vocab_size, self.hidden_size))}
 
     def load(self, tensors, build: BuildContext) -> None:
-        self.weight = tensors["weight"].contiguous()
+        self.weight = tensors[self.tensor].contiguous()
 
     def forward(self, tokens: torch.Tensor) -> torch.Tensor:
         """The residual stream of the step's tokens, float32 ``[n, d]``."""
         out = torch.empty((tokens.numel(), self.hidden_size), dtype=torch.float32, device=tokens.device)
-        return ops.embedding_gather(self.weight, tokens, out)
+        return ops.embedding_gather(self.weight, tokens, out, self.scale)
 
 
 class OutputHead(Part):
@@ -43,17 +46,18 @@ class OutputHead(Part):
 
     """``logits = y @ W.T``; ``tied``: W is the embedding table."""
 
-    def __init__(self, vocab_size: int, hidden_size: int, tied: bool = False):
+    def __init__(self, vocab_size: int, hidden_size: int, tied: bool = False, tensor: str = "weight"):
         self.vocab_size, self.hidden_size, self.tied = int(vocab_size), int(hidden_size), bool(tied)
+        self.tensor = str(tensor)
         self.weight = None
 
     def tensors(self):
         # a file may hold the matrix although the model ties it (then it is not used), or
         # hold none although it does not (then the table is used: the reference's rule)
-        return {"weight": TensorSpec((self.vocab_size, self.hidden_size), optional=True, random=not self.tied)}
+        return {self.tensor: TensorSpec((self.vocab_size, self.hidden_size), optional=True, random=not self.tied)}
 
     def load(self, tensors, build: BuildContext, table: Optional[torch.Tensor] = None) -> None:
-        own = tensors.get("weight")
+        own = tensors.get(self.tensor)
         self.weight = Weight(table if (self.tied or own is None) else own, build)
         self.dtype = build.dtype
 
@@ -123,6 +127,10 @@ class DecoderModel:
                 part.load(mine, build)
 
     # ---- caches
+    def own_states(self):
+        """For every entry of the run order: the states that its layer's block keeps itself (``Part.own_states``)."""
+        return [self.layers[e.layer].own_states() for e in self.spec.run_order]
+
     def cache_needs(self):
         """For every entry of the run order: the need of its layer's mixer, or None if it
         reads another entry's cache (or needs none)."""

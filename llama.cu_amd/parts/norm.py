@@ -1,4 +1,4 @@
-"""RMS normalisation, fused with the residual sum that precedes it.
+"""RMS normalisation and layer normalisation, fused with the residual sum that precedes them.
 
 ``y = x * rsqrt(sum(x^2)/d + eps) * w`` (llama.cu/src/op/rms_norm.cuh:21-29), in
 32-bit with one rounding at the store; the weight may be stored in another type than
@@ -48,4 +48,33 @@ class RMSNorm(Part):
     takes_planes = True
 
 
+class LayerNorm(Part):
+    """``y = (x - mean(x)) * rsqrt(var(x) + eps) * w + b`` with the variance as the mean of the squared deviations,
+    in 32-bit.  ``tensor`` and ``bias_tensor`` name its two tensors (files of different designs name them
+    differently).  ``forward`` may be asked for 32-bit output (``out_dtype``) by a block that goes on in 32-bit."""
+    graph_safe = True
+    takes_planes = True        # delta may be float32 planes [planes, n, d], added one after the other
+
+    def __init__(self, size: int, eps: float, tensor: str = "weight", bias_tensor: str = "bias"):
+        self.size, self.eps = int(size), float(eps)
+        self.tensor, self.bias_tensor = str(tensor), str(bias_tensor)
+        self.weight = self.bias = None
+        self.dtype = None
+
+    def tensors(self) -> Dict[str, TensorSpec]:
+        return {self.tensor: TensorSpec((self.size,), init="one_plus_normal"),
+                self.bias_tensor: TensorSpec((self.size,), init="normal")}
+
+    def load(self, tensors, build: BuildContext) -> None:
+        # the kernels take the two vectors in 32-bit whatever the file holds
+        self.weight = tensors[self.tensor].float().contiguous()
+        self.bias = tensors[self.bias_tensor].float().contiguous()
+        self.dtype = build.dtype
+
+    def forward(self, x: torch.Tensor, delta: Optional[torch.Tensor] = None, out_dtype=None) -> torch.Tensor:
+        out = torch.empty(x.shape, dtype=out_dtype or self.dtype, device=x.device)
+        return ops.layernorm(x, self.weight, self.bias, self.eps, out, delta=delta)
+
+
 register_part("norm", "rmsnorm", RMSNorm)
+register_part("norm", "layernorm", LayerNorm)

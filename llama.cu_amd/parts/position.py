@@ -97,5 +97,24 @@ class Rotary(NoPosition):
         return self.cos, self.sin, self.rot_dim, 1 if self.interleaved else 0
 
 
+class DistanceBias(NoPosition):
+    """No change of queries and keys: the scaled score of key ``j`` for the query at ``i`` of head ``h`` is lowered
+    by ``slope[h] * (i - j)`` with ``slope[h] = 2^(-exponent * (h + 1) / heads)``, ``h = 0 .. heads - 1``."""
+
+    def __init__(self, heads: int, exponent: float = 8.0):
+        self.heads, self.exponent = int(heads), float(exponent)
+        self.slopes = None
+
+    def host_slopes(self):
+        return np.array([2.0 ** (-self.exponent * (h + 1) / self.heads) for h in range(self.heads)], dtype=np.float32)
+
+    def load(self, tensors, build: BuildContext) -> None:
+        self.slopes = torch.from_numpy(self.host_slopes()).to(build.device).contiguous()
+
+    def score_slopes(self):
+        return self.slopes
+
+
 register_part("position", "none", NoPosition)
+register_part("position", "distance_bias", DistanceBias)
 register_part("position", "rotary", Rotary)
