@@ -1007,7 +1007,7 @@ def short_conv(h: torch.Tensor, weight: torch.Tensor, state: torch.Tensor, out: 
     taps = weight.shape[2]
     if state.dtype != torch.float32 or state.dim() != 4 or state.shape[1:] != (sets, taps - 1, d):
         raise KernelError(f"short_conv: state must be float32 [slots, {sets}, {taps - 1}, {d}], got {state.dtype} {tuple(state.shape)}")
-    if n != step.n or max(step.state_slots, default=0) >= state.shape[0]:
+    if n != step.n or (taps > 1 and max(step.state_slots, default=0) >= state.shape[0]):
         raise KernelError("short_conv: the rows are not the step's, or a request's slot lies outside the state")
     lib = build.load("norm_conv")
     _check(lib.lcu_short_conv(_ptr(h), _type(h, "conv input"), ctypes.c_longlong(n * d), _ptr(weight), _type(weight, "conv weight"),

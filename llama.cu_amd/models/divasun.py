@@ -58,5 +58,6 @@ def divasun_spec(cfg: DivasunConfig) -> ModelSpec:
         eos_token_ids=cfg.eos_token_ids)
 
 
-register_architecture("Divasun", DivasunConfig.from_dict, divasun_spec,
+# a file may hold the second norm and its convolution also for a layer that has no feed-forward to read them
+register_architecture("Divasun", DivasunConfig.from_dict, divasun_spec, ignored_tensors=[r"l\d+\.(norm2|norm2\.b|canon2)$"],
                       complete_config=lambda cfg, shapes: cfg.complete_from_shapes(shapes))

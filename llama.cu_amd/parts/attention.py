@@ -36,9 +36,9 @@ class Attention(Part):
         position ``p`` is multiplied by ``1 + coef * ln(floor((p + 1) / every) + 1)``."""
         if heads % kv_heads:
             raise ValueError(f"attention: {heads} heads are no multiple of {kv_heads} key/value heads")
-        if head_dim % 16 or head_dim > 256:
+        if head_dim % 8 or head_dim > 256:
             raise ValueError(f"attention: head_dim {head_dim} is not supported by the kernels "
-                             f"(multiples of 16 up to 256)")
+                             f"(multiples of 8 up to 256)")
         self.hidden_size, self.heads, self.kv_heads, self.head_dim = int(hidden_size), int(heads), int(kv_heads), int(head_dim)
         self.scale = float(scale) if scale is not None else float(head_dim) ** -0.5
         self.window = int(window or 0)

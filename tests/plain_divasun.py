@@ -98,9 +98,14 @@ def attention(h, P, heads: int, kv_heads: int, dim: int, vdim: int, scale: float
     return out.reshape(T, heads * vdim) @ P["o"].T
 
 
-def moe(h, P, experts: int, top: int):
-    """Every token's ``top`` experts by sigmoid score; the score multiplies the expert's input."""
-    s = torch.sigmoid(h @ P["router"].T)
+def moe(h, P, experts: int, top: int, margins: Optional[list] = None):
+    """Every token's ``top`` experts by sigmoid score; the score multiplies the expert's input.  ``margins`` takes
+    every token's distance between the last chosen logit and the first that was not (how close the call was)."""
+    z = h @ P["router"].T
+    s = torch.sigmoid(z)
+    if margins is not None and top < experts:
+        ranked = torch.sort(z, dim=-1, descending=True).values
+        margins.extend((ranked[:, top - 1] - ranked[:, top]).tolist())
     out = torch.zeros(h.shape[0], P["e0.down"].shape[0], dtype=h.dtype)
     order = torch.argsort(-s, dim=-1, stable=True)[:, :top]
     for t in range(h.shape[0]):
@@ -114,7 +119,8 @@ def sub(tensors: Dict[str, torch.Tensor], prefix: str) -> Dict[str, torch.Tensor
     return {k[len(prefix):]: v for k, v in tensors.items() if k.startswith(prefix)}
 
 
-def forward(cfg: dict, tensors: Dict[str, torch.Tensor], tokens: List[int], layers_out: Optional[list] = None):
+def forward(cfg: dict, tensors: Dict[str, torch.Tensor], tokens: List[int], layers_out: Optional[list] = None,
+            margins: Optional[list] = None):
     """Logits ``[T, vocab]`` of one whole sequence from position 0."""
     W = {k: (v.to(F) if v.is_floating_point() else v) for k, v in tensors.items()}
     eps = cfg["norm"]["eps"]
@@ -140,7 +146,7 @@ def forward(cfg: dict, tensors: Dict[str, torch.Tensor], tokens: List[int], laye
         if layer.get("mlp") is not None:
             h2 = short_conv(layer_norm(x, W[pre + "norm2"], W[pre + "norm2.b"], eps), W[pre + "canon2"])
             f = layer["mlp"]
-            a = a + moe(h2, sub(W, pre + "mlp."), f["router"]["experts"], f["router"]["top"])
+            a = a + moe(h2, sub(W, pre + "mlp."), f["router"]["experts"], f["router"]["top"], margins)
         x = x + a
         if layers_out is not None:
             layers_out.append(x.clone())
