@@ -334,6 +334,83 @@ def library_product(cfg, sync, calls=400):
     return out
 
 
+# ---------------------------------------------------------------------------- --workload designs
+# Layer sizes at which the Divasun design is measured beside the Llama dense decoder: the same width, layers, heads and
+# head size, and a feed-forward of the same number of active weights (top * 2 * width * ff = 3 * width * intermediate).
+DESIGN_SIZES = {
+    "w2048": dict(width=2048, layers=8, heads=16, kv_heads=4, dim=128, experts=16, top=2, ff=2048, vocab=32000),
+    "w4096": dict(width=4096, layers=4, heads=32, kv_heads=8, dim=128, experts=16, top=4, ff=5376, vocab=32000),
+}
+
+
+def divasun_config(z, positions):
+    """Delta rule and attention in turn; the last attention layer reads the keys and values of the one before it."""
+    from llama_cu_amd.config import DivasunConfig
+    layers, last_attention = [], None
+    for i in range(z["layers"]):
+        mlp = {"kind": "moe", "router": {"experts": z["experts"], "top": z["top"]}, "expert": {"ff": z["ff"]}}
+        if i % 2 == 0:
+            layers.append({"type": "general_delta", "mixer": {"heads": z["heads"], "dim": z["dim"], "decay_rank": 64}, "mlp": mlp})
+        else:
+            m = {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["dim"], "vdim": z["dim"], "scale": z["dim"] ** -0.5,
+                 "q_temp": {"coef": 0.3, "every": 256}}
+            if i == z["layers"] - 1 and last_attention is not None:
+                m["kv_from"] = last_attention
+            else:
+                last_attention = i
+            layers.append({"type": "attention", "mixer": m, "mlp": mlp})
+    return DivasunConfig.from_dict({"architecture": "Divasun", "vocab": z["vocab"], "width": z["width"], "layers": layers,
+                                    "norm": {"eps": 1e-5}, "canon": {"taps": 4}, "embedding": {"scale": z["width"] ** 0.5},
+                                    "max_positions": positions})
+
+
+def llama_like(z, positions):
+    from llama_cu_amd.config import LlamaConfig
+    inter = (z["top"] * 2 * z["ff"] // 3 + 127) // 128 * 128
+    return LlamaConfig.from_dict(dict(SHAPE, num_hidden_layers=z["layers"], hidden_size=z["width"], num_attention_heads=z["heads"],
+                                      num_key_value_heads=z["kv_heads"], head_dim=z["dim"], intermediate_size=inter,
+                                      vocab_size=z["vocab"], max_position_embeddings=positions))
+
+
+def run_designs(args):
+    """Prefill (one step of 2,048 tokens) and decode (8 and 64 requests over prompts of 512 tokens) throughput of the
+    Divasun design beside the Llama dense decoder at equal layer sizes, random weights; one JSON line."""
+    import gc
+
+    import torch
+    import llama_cu_amd  # noqa: F401
+    from llama_cu_amd.engine.engine import Engine
+    sync = torch.cuda.synchronize
+    page, prompt, positions = args.page_size, 512, 4096
+    steps, warmup = min(args.steps, 32), min(args.warmup, 8)
+    rows = []
+    for name, z in DESIGN_SIZES.items():
+        for design, cfg in (("divasun", divasun_config(z, positions)), ("llama", llama_like(z, positions))):
+            rng = random.Random(0)
+            biggest = 64
+            per_req = prompt + steps + warmup + 2 * biggest + 72
+            engine = Engine.from_config(cfg, seed=0, dtype=args.dtype, page_size=page,
+                                        max_tokens=biggest * ((per_req + page - 1) // page * page) + PREFILL_TOKENS + page,
+                                        max_seqs=biggest + 2, max_batch_tokens=PREFILL_TOKENS, prefill_chunk=PREFILL_TOKENS)
+            vocab = cfg.vocab if design == "divasun" else cfg.vocab_size
+            shim = type("V", (), {"vocab_size": vocab})
+            pt = run_prefill(engine, shim, rng, sync)
+            row = {"size": name, "design": design, "prefill_tok_s": round(PREFILL_TOKENS / pt, 1), "prefill_ms": round(pt * 1e3, 3)}
+            for b in (8, 64):
+                sec, produced, _ = run_decode(engine, shim, b, steps, warmup, rng, sync, prompt_len=prompt)
+                row[f"decode_b{b}_tok_s"] = round(produced / sec, 1)
+                row[f"decode_b{b}_ms_per_step"] = round(run_decode.median_ms, 4)
+            rows.append(row)
+            print(f"[bench] {row}", file=sys.stderr, flush=True)
+            del engine
+            gc.collect()
+            torch.cuda.empty_cache()
+    print(json.dumps({"metric": "prefill and decode throughput of two designs at equal layer sizes", "unit": "tok/s", "n_gpus": 1,
+                      "dtype": "bf16" if args.dtype == "bfloat16" else "f32", "data": "synthetic", "steps": steps, "warmup": warmup,
+                      "sizes": DESIGN_SIZES, "rows": rows}), flush=True)
+    return 0
+
+
 def kernel_summary(db: str, steps: int, launches: int = 0) -> int:
     """Per-step table of kernels from the database that ``rocprofv3 --kernel-trace`` wrote for a
     run of this program: the kernels between two embedding gathers are one step of the model;
@@ -381,7 +458,7 @@ def main() -> int:
                          "limit grows with it)")
     ap.add_argument("--dtype", choices=["bfloat16", "float32"], default="bfloat16")
     ap.add_argument("--page-size", type=int, default=16, help="tokens in a page of the cache (a multiple of 16)")
-    ap.add_argument("--workload", choices=["decode", "mixed", "arrivals"], default="decode",
+    ap.add_argument("--workload", choices=["decode", "mixed", "arrivals", "designs"], default="decode",
                     help="decode: --batch requests decode together after prompts of --prompt-len (the default); mixed: "
                          "--batch requests at once with prompt lengths uniform in [16, 2048], 128 tokens each, through the "
                          "scheduler (the workload that goes with --shape llama2-7b --batch 64); arrivals: --batch requests "
@@ -409,6 +486,8 @@ def main() -> int:
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported (no multi-GPU path)")
         return 2
+    if args.workload == "designs":
+        return run_designs(args)
 
     import torch
     import llama_cu_amd  # noqa: F401
