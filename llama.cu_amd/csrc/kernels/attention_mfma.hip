@@ -45,12 +45,31 @@ __device__ __forceinline__ f32x4 mfma16(u32x4 a, u32x4 b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
 }
 
+// LCU_SCORE_BIAS (defined by the file that includes this one to build the second library): every kernel and entry
+// point takes head_slopes [nh] as well, and slope[h] * (j - p) is added to the scaled score of key j for the query at
+// position p of head h (a bias that grows with the distance).  Inside the kernels the bias stands in the scores' own
+// units (slope / scale), so that everything after the scores is the same code.
+#ifdef LCU_SCORE_BIAS
+#define BIAS_KPARAMS , const float *__restrict__ head_slopes, float inv_scale
+#define BIAS_KARGS(scale) , head_slopes, 1.0f / (scale)
+#define BIAS_PARAMS , const float *head_slopes
+#define BIAS_ARGS , head_slopes
+#else
+#define BIAS_KPARAMS
+#define BIAS_KARGS(scale)
+#define BIAS_PARAMS
+#define BIAS_ARGS
+#endif
+
 // What a wave carries through its keys, for QB blocks of 16 rows.
 template <int DH, int QB>
 struct AttnState {
     f32x4 o[QB][DH / 16];   // O^T: lane = (row lane%16, dims 16*dt + 4*(lane/16) + r)
     float m[QB];            // running maximum (in units of log2), the same in the 4 lane groups
     float l[QB];            // running sum over the lane's own keys only
+#ifdef LCU_SCORE_BIAS
+    float bias[QB];         // of the lane's row: slope of its head / scale
+#endif
 };
 
 template <int DH, int QB>
@@ -59,6 +78,9 @@ __device__ __forceinline__ void attn_init(AttnState<DH, QB> &st) {
     for (int b = 0; b < QB; ++b) {
         st.m[b] = -INFINITY;
         st.l[b] = 0.f;
+#ifdef LCU_SCORE_BIAS
+        st.bias[b] = 0.f;
+#endif
 #pragma unroll
         for (int dt = 0; dt < DH / 16; ++dt) st.o[b][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
@@ -183,6 +205,10 @@ __device__ __forceinline__ void attn_softmax(const f32x4 (&s)[QB][2], int k0, At
         float v[8];
 #pragma unroll
         for (int r = 0; r < 4; ++r) { v[r] = s[b][0][r]; v[4 + r] = s[b][1][r]; }
+#ifdef LCU_SCORE_BIAS
+#pragma unroll
+        for (int r = 0; r < 8; ++r) v[r] = fmaf(st.bias[b], (float)(k0 + 16 * (r / 4) + 4 * grp + (r % 4) - p_row[b]), v[r]);
+#endif
         if (MASK) {
 #pragma unroll
             for (int r = 0; r < 8; ++r) {
@@ -285,7 +311,7 @@ attention_decode_kernel(const bf16_t *__restrict__ q, int q_stride, bf16_t *__re
                         const bf16_t *__restrict__ cache, const int *__restrict__ block_table, int max_pages,
                         const int *__restrict__ q_start, const int *__restrict__ ctx_len,
                         const int *__restrict__ req_list, int nh, int nkvh, int page, float scale_log2, int window,
-                        int n_splits, float *__restrict__ part_o, float *__restrict__ part_ml) {
+                        int n_splits, float *__restrict__ part_o, float *__restrict__ part_ml BIAS_KPARAMS) {
     extern __shared__ float lds[];                 // [waves][16][DH] outputs, then [waves][16][2] (m, l)
     const int g = nh / nkvh;
     const int chunks = (g + 15) / 16;
@@ -308,6 +334,9 @@ attention_decode_kernel(const bf16_t *__restrict__ q, int q_stride, bf16_t *__re
     load_q<DH>(q + (size_t)token * q_stride + (size_t)(head0 + l16) * DH, l16 < rows, qv[0], grp);
     AttnState<DH, 1> st;
     attn_init(st);
+#ifdef LCU_SCORE_BIAS
+    st.bias[0] = l16 < rows ? head_slopes[head0 + l16] * inv_scale : 0.f;
+#endif
     const int p_row[1] = {p}, lo_row[1] = {lo};
     const int *bt = block_table + (size_t)r * max_pages;
     const size_t page_elems = kv_page_elems(nkvh, DH, page);
@@ -442,7 +471,7 @@ template <int DH>
 static int launch_decode(const void *q, int q_stride, void *out, int out_stride, const void *cache,
                          const int *block_table, int max_pages, const int *q_start, const int *ctx_len,
                          const int *req_list, int n_req, int nh, int nkvh, int page, float scale, int window,
-                         int n_splits, float *part_o, float *part_ml, hipStream_t stream) {
+                         int n_splits, float *part_o, float *part_ml, hipStream_t stream BIAS_PARAMS) {
     const int g = nh / nkvh, chunks = (g + 15) / 16;
     const float scale_log2 = scale * 1.4426950408889634f;
     const size_t lds_bytes = (size_t)DEC_WAVES * 16 * (DH + 2) * sizeof(float);
@@ -456,7 +485,7 @@ static int launch_decode(const void *q, int q_stride, void *out, int out_stride,
     const bool flat = n_splits == 1;
     (flat ? attention_decode_kernel<DH, true> : attention_decode_kernel<DH, false>)<<<grid, block, lds_bytes, stream>>>(
         (const bf16_t *)q, q_stride, (bf16_t *)out, out_stride, (const bf16_t *)cache, block_table, max_pages, q_start,
-        ctx_len, req_list, nh, nkvh, page, scale_log2, window, n_splits, part_o, part_ml);
+        ctx_len, req_list, nh, nkvh, page, scale_log2, window, n_splits, part_o, part_ml BIAS_KARGS(scale));
     LCU_LAUNCH_CHECK();
     if (n_splits > 1) {
         attention_merge_kernel<DH><<<dim3(n_req, nh), dim3(DH / 4), 0, stream>>>((bf16_t *)out, out_stride, part_o, part_ml,
@@ -484,12 +513,15 @@ static int decode_arguments(int q_stride, int out_stride, int max_pages, int nh,
 LCU_API int lcu_attention_decode_bf16(const void *q, int q_stride, void *out, int out_stride, const void *cache,
                                       const int *block_table, int max_pages, const int *q_start, const int *ctx_len,
                                       const int *req_list, int n_req, int nh, int nkvh, int dh, int page, float scale,
-                                      int window, int n_splits, float *part_o, float *part_ml, hipStream_t stream) {
+                                      int window, int n_splits, float *part_o, float *part_ml, hipStream_t stream BIAS_PARAMS) {
     if (n_req <= 0) return LCU_OK;
+#ifdef LCU_SCORE_BIAS
+    if (!head_slopes || !(scale > 0.f)) return LCU_BAD_ARGUMENT;
+#endif
     const int args = decode_arguments(q_stride, out_stride, max_pages, nh, nkvh, dh, page, window, n_splits);
     if (args != LCU_OK) return args;
     if (n_splits > 1 && (!part_o || !part_ml)) return LCU_BAD_ARGUMENT;
-#define GO(D) return launch_decode<D>(q, q_stride, out, out_stride, cache, block_table, max_pages, q_start, ctx_len, req_list, n_req, nh, nkvh, page, scale, window, n_splits, part_o, part_ml, stream)
+#define GO(D) return launch_decode<D>(q, q_stride, out, out_stride, cache, block_table, max_pages, q_start, ctx_len, req_list, n_req, nh, nkvh, page, scale, window, n_splits, part_o, part_ml, stream BIAS_ARGS)
     if (dh == 128) GO(128);
     if (dh == 64) GO(64);
     if (dh == 96) GO(96);
@@ -542,6 +574,9 @@ LCU_API int lcu_attention_decode_bf16_static(const void *q, int q_stride, void *
                                              const int *block_table, int max_pages, const int *q_start, const int *ctx_len,
                                              const int *req_list, int n_req, int nh, int nkvh, int dh, int page, float scale,
                                              int window, int n_splits, hipStream_t stream) {
+#ifdef LCU_SCORE_BIAS
+    return LCU_UNSUPPORTED;        // (this entry point takes no slopes: the library with the bias has no such caller)
+#else
     if (n_req <= 0) return LCU_OK;
     // the arguments first, as the other entry point checks them: a call with bad sizes is told so, whatever
     // buffer it would need
@@ -559,6 +594,7 @@ LCU_API int lcu_attention_decode_bf16_static(const void *q, int q_stride, void *
     }
     return lcu_attention_decode_bf16(q, q_stride, out, out_stride, cache, block_table, max_pages, q_start, ctx_len, req_list,
                                      n_req, nh, nkvh, dh, page, scale, window, n_splits, part_o, part_ml, stream);
+#endif
 }
 
 // ============================================================================ prefill
@@ -600,6 +636,9 @@ struct PrefillState {
     f32x16 o[DH / 32];      // O^T: lane = (row lane % 32, dims 32 t + 8 (i / 4) + 4 hi + i % 4)
     float m;                // running maximum (in units of log2), the same in the row's two lanes
     float l;                // running sum over the lane's own keys only
+#ifdef LCU_SCORE_BIAS
+    float bias;             // of the lane's row: slope of its head / scale (0 for a row that is nobody's)
+#endif
 };
 
 // The larger of the values that lane l and lane l ^ 32 hold, in both.
@@ -823,6 +862,15 @@ __device__ __forceinline__ void attn_turn(const u32x4 *__restrict__ next, u32x4 
     float x[16];
 #pragma unroll
     for (int i = 0; i < 16; ++i) x[i] = s[i];
+#ifdef LCU_SCORE_BIAS
+    {
+        // the lane's score i is key k0 + 8 hi + c with c = 16 (i / 8) + i % 8, so its distance to the row's position
+        // is c - (p_row - k0 - 8 hi); a turn that is not the wave's own (p_row = -1) masks everything below
+        const int last0 = p_row - k0 - 8 * hi;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) x[i] = fmaf(st.bias, (float)(16 * (i / 8) + i % 8 - last0), x[i]);
+    }
+#endif
     if (mask) {
         // a lane's score i is key k0 + 8 hi + c with c = 16 (i / 8) + i % 8: compared as c against the bounds less k0 + 8 hi
         const int last = p_row - k0 - 8 * hi, first = lo_row - k0 - 8 * hi;
@@ -892,7 +940,7 @@ attention_prefill_kernel(const bf16_t *__restrict__ q, int q_stride, bf16_t *__r
                            const int *__restrict__ q_start, const int *__restrict__ ctx_len,
                            const int *__restrict__ task_req, const int *__restrict__ task_tok0, int max_tasks,
                            const int *__restrict__ n_tasks_dev,
-                           int tasks_per_wg, int nh, int nkvh, int page, uint32_t tile_magic, float scale_log2, int window) {
+                           int tasks_per_wg, int nh, int nkvh, int page, uint32_t tile_magic, float scale_log2, int window BIAS_KPARAMS) {
     extern __shared__ u32x4 lds_ring[];            // [PRE_RING][8 * DH]
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
     const int lane = threadIdx.x & (WAVE - 1);
@@ -947,6 +995,9 @@ attention_prefill_kernel(const bf16_t *__restrict__ q, int q_stride, bf16_t *__r
     PrefillState<DH> st;
     st.m = -INFINITY;
     st.l = 0.f;
+#ifdef LCU_SCORE_BIAS
+    st.bias = valid ? head_slopes[head0 + n % hc] * inv_scale : 0.f;
+#endif
 #pragma unroll
     for (int t = 0; t < DH / 32; ++t)
 #pragma unroll
@@ -1038,7 +1089,7 @@ template <int DH, bool PAGE16, bool FLAT>
 static int launch_prefill_as(const void *q, int q_stride, void *out, int out_stride, const void *cache, uint32_t cache_bytes,
                              const int *block_table, int max_pages, const int *q_start, const int *ctx_len,
                              const int *task_req, const int *task_tok0, int n_tasks, const int *n_tasks_dev, int tasks_per_wg,
-                             int nh, int nkvh, int page, float scale, int window, hipStream_t stream) {
+                             int nh, int nkvh, int page, float scale, int window, hipStream_t stream BIAS_PARAMS) {
     const int g = nh / nkvh, chunks = (g + 15) / 16;
     const long long n_wg = (long long)((n_tasks + tasks_per_wg - 1) / tasks_per_wg) * nkvh * chunks;
     if (n_wg > 0x7fffffffll) return LCU_BAD_ARGUMENT;
@@ -1061,7 +1112,7 @@ static int launch_prefill_as(const void *q, int q_stride, void *out, int out_str
     attention_prefill_kernel<DH, PAGE16, FLAT><<<grid, block, lds_bytes, stream>>>(
         (const bf16_t *)q, q_stride, (bf16_t *)out, out_stride, (const bf16_t *)cache, cache_bytes, block_table, max_pages, q_start,
         ctx_len, task_req, task_tok0, n_tasks, n_tasks_dev, tasks_per_wg, nh, nkvh, page,
-        page == 16 ? 0u : (uint32_t)(0x100000000ull / (unsigned)(page / 16)) + 1u, scale * 1.4426950408889634f, window);
+        page == 16 ? 0u : (uint32_t)(0x100000000ull / (unsigned)(page / 16)) + 1u, scale * 1.4426950408889634f, window BIAS_KARGS(scale));
     LCU_LAUNCH_CHECK();
     return LCU_OK;
 }
@@ -1071,10 +1122,10 @@ template <int DH>
 static int launch_prefill(const void *q, int q_stride, void *out, int out_stride, const void *cache, long long cache_pages,
                           const int *block_table, int max_pages, const int *q_start, const int *ctx_len,
                           const int *task_req, const int *task_tok0, int n_tasks, const int *n_tasks_dev, int tasks_per_wg,
-                          int nh, int nkvh, int page, float scale, int window, hipStream_t stream) {
+                          int nh, int nkvh, int page, float scale, int window, hipStream_t stream BIAS_PARAMS) {
     const unsigned long long bytes = (unsigned long long)cache_pages * kv_page_elems(nkvh, DH, page) * sizeof(bf16_t);
     const bool flat = bytes < (1ull << 32);
-#define AS(P, F) return launch_prefill_as<DH, P, F>(q, q_stride, out, out_stride, cache, (uint32_t)(F ? bytes : 0), block_table, max_pages, q_start, ctx_len, task_req, task_tok0, n_tasks, n_tasks_dev, tasks_per_wg, nh, nkvh, page, scale, window, stream)
+#define AS(P, F) return launch_prefill_as<DH, P, F>(q, q_stride, out, out_stride, cache, (uint32_t)(F ? bytes : 0), block_table, max_pages, q_start, ctx_len, task_req, task_tok0, n_tasks, n_tasks_dev, tasks_per_wg, nh, nkvh, page, scale, window, stream BIAS_ARGS)
     if (page == 16) {
         if (flat) AS(true, true);
         AS(true, false);
@@ -1103,13 +1154,16 @@ LCU_API int lcu_attention_prefill_bf16(const void *q, int q_stride, void *out, i
                                        long long cache_pages, const int *block_table, int max_pages, const int *q_start, const int *ctx_len,
                                        const int *task_req, const int *task_tok0, int n_tasks, const int *n_tasks_dev,
                                        int tasks_per_wg, int nh, int nkvh, int dh, int page, float scale, int window,
-                                       hipStream_t stream) {
+                                       hipStream_t stream BIAS_PARAMS) {
     if (n_tasks <= 0) return LCU_OK;
+#ifdef LCU_SCORE_BIAS
+    if (!head_slopes || !(scale > 0.f)) return LCU_BAD_ARGUMENT;
+#endif
     if ((unsigned long long)kv_page_elems(nkvh, dh, page) * 2ull >= (1ull << 31)) return LCU_UNSUPPORTED;
     if (cache_pages <= 0 || tasks_per_wg < 1 || lcu_attention_prefill_tokens_per_task(nh, nkvh) == 0 || page <= 0 || page % 16 || max_pages <= 0 ||
         window < 0 || q_stride % 8 || out_stride % 4 || nkvh * ((nh / nkvh + 15) / 16) > 65535)
         return LCU_BAD_ARGUMENT;
-#define GO(D) return launch_prefill<D>(q, q_stride, out, out_stride, cache, cache_pages, block_table, max_pages, q_start, ctx_len, task_req, task_tok0, n_tasks, n_tasks_dev, tasks_per_wg, nh, nkvh, page, scale, window, stream)
+#define GO(D) return launch_prefill<D>(q, q_stride, out, out_stride, cache, cache_pages, block_table, max_pages, q_start, ctx_len, task_req, task_tok0, n_tasks, n_tasks_dev, tasks_per_wg, nh, nkvh, page, scale, window, stream BIAS_ARGS)
     if (dh == 128) GO(128);
     if (dh == 64) GO(64);
     if (dh == 96) GO(96);

@@ -9,8 +9,8 @@
 //           w = exp(-exp(-1/2) * sigmoid(w0 + W2 tanh(l))), l the row's low-rank projection,
 //           a = sigmoid(a_lin + a_bias);
 //   scan  (sequential over a request's tokens, parallel over requests, heads and value
-//           channels: column j of S depends on column j alone, so a lane owns a column and
-//           keeps it in registers from the request's first token of the step to its last);
+//           channels: column j of S depends on column j alone, so a column stays in the registers
+//           of its lanes from the request's first token of the step to its last);
 //   out   (parallel): o of each head divided by its root mean square, times a weight, times
 //           sigmoid(gate).
 // A token's result depends on the tokens before it in its request only, in an order of
@@ -57,76 +57,101 @@ __global__ void delta_prep_kernel(const T *__restrict__ proj, int row_stride, in
     }
 }
 
-// One wave per (request, head, 64 value channels).  DK > 0: the column of S lives in DK
-// registers; DK == 0: any dk, the column stays in the state's memory.
+// DK > 0 (a multiple of 16): one wave per (request, head, 16 value channels).  The wave's lanes are four groups of 16:
+// lane (g, j) keeps the quarter g of column j of S (key channels g * DK/4 .. + DK/4 - 1) in registers, so a token
+// costs a lane DK/4 of each pass, and the two sums over key channels (u^T S and S^T r) cross the groups with two
+// shuffles each.  The token's five vectors go through LDS (all lanes copy, each reads its quarter), the next
+// token's are on their way meanwhile.
+// DK == 0: any dk, one wave per (request, head, 64 value channels), the column stays in the state's memory.
 // state: [slots, heads, dk, dv]; o: [n, heads * dv] 32-bit.
+constexpr int SCAN_GROUPS = 4, SCAN_COLS = WAVE / SCAN_GROUPS;
+
 template <class T, int DK>
 __global__ void __launch_bounds__(64)
 delta_scan_kernel(const T *__restrict__ proj, int row_stride, int off_v, const float *__restrict__ prep,
                   float *__restrict__ state, float *__restrict__ o, const int *__restrict__ q_start,
                   const int *__restrict__ ctx_len, const int *__restrict__ state_slot, int heads, int dk_rt, int dv) {
-    const int dk = DK > 0 ? DK : dk_rt;
-    const int r = blockIdx.x, h = blockIdx.y, j = blockIdx.z * 64 + threadIdx.x;
+    const int r = blockIdx.x, h = blockIdx.y;
     const int t0 = q_start[r], t1 = q_start[r + 1];
     const bool fresh = ctx_len[r] - (t1 - t0) == 0;          // the request's first token: the state starts at zero
-    const bool live = j < dv;
-    const int jj = live ? j : dv - 1;                        // lanes beyond dv compute along and store nothing
-    float *col = state + (((size_t)state_slot[r] * heads + h) * dk) * dv + jj;     // S[i][j] at col[i * dv]
-    __shared__ float vec[2][5 * (DK > 0 ? DK : 1)];
-    float S[DK > 0 ? DK : 1];
-    if (DK > 0) {
+    if constexpr (DK > 0) {
+        constexpr int SL = DK / SCAN_GROUPS;                  // key channels of a lane
+        constexpr int PER_LANE = (5 * DK + 63) / 64;
+        const int g = threadIdx.x / SCAN_COLS, j = blockIdx.z * SCAN_COLS + threadIdx.x % SCAN_COLS;
+        const bool live = j < dv;
+        const int jj = live ? j : dv - 1;                     // lanes beyond dv compute along and store nothing
+        float *col = state + (((size_t)state_slot[r] * heads + h) * DK + g * SL) * dv + jj;   // S[g * SL + i][j] at col[i * dv]
+        __shared__ __attribute__((aligned(16))) float vec[2][5 * DK];
+        float S[SL];
 #pragma unroll
-        for (int i = 0; i < DK; ++i) S[i] = fresh ? 0.f : col[(size_t)i * dv];
-    } else if (fresh && live) {
-        for (int i = 0; i < dk; ++i) col[(size_t)i * dv] = 0.f;
-    }
-    constexpr int PER_LANE = DK > 0 ? (5 * DK + 63) / 64 : 1;
-    float next[PER_LANE];
-    auto fetch = [&](int t) {
-        const float *p = prep + ((size_t)t * heads + h) * 5 * dk;
+        for (int i = 0; i < SL; ++i) S[i] = fresh ? 0.f : col[(size_t)i * dv];
+        float next[PER_LANE];
+        auto fetch = [&](int t) {
+            const float *p = prep + ((size_t)t * heads + h) * 5 * DK;
 #pragma unroll
-        for (int e = 0; e < PER_LANE; ++e) {
-            const int idx = e * 64 + threadIdx.x;
-            next[e] = idx < 5 * dk ? p[idx] : 0.f;
+            for (int e = 0; e < PER_LANE; ++e) {
+                const int idx = e * 64 + threadIdx.x;
+                next[e] = idx < 5 * DK ? p[idx] : 0.f;
+            }
+        };
+        const T *vp = proj + off_v + h * dv + jj;
+        float v_next = 0.f;
+        if (t0 < t1) {
+            fetch(t0);
+            v_next = to_f32(vp[(size_t)t0 * row_stride]);
         }
-    };
-    if (DK > 0 && t0 < t1) fetch(t0);
-    for (int t = t0; t < t1; ++t) {
-        const float v = to_f32(proj[(size_t)t * row_stride + off_v + h * dv + jj]);
-        float acc = 0.f;
-        if (DK > 0) {
+        for (int t = t0; t < t1; ++t) {
             float *cur = vec[(t - t0) & 1];
 #pragma unroll
             for (int e = 0; e < PER_LANE; ++e) {
                 const int idx = e * 64 + threadIdx.x;
                 if (idx < 5 * DK) cur[idx] = next[e];
             }
+            const float v = v_next;
             __syncthreads();
-            if (t + 1 < t1) fetch(t + 1);
-            const float *W = cur, *AU = cur + DK, *U = cur + 2 * DK, *K = cur + 3 * DK, *R = cur + 4 * DK;
+            if (t + 1 < t1) {
+                fetch(t + 1);
+                v_next = to_f32(vp[(size_t)(t + 1) * row_stride]);
+            }
+            const float *W = cur + g * SL, *AU = W + DK, *U = W + 2 * DK, *K = W + 3 * DK, *R = W + 4 * DK;
             float us = 0.f;
 #pragma unroll
-            for (int i = 0; i < DK; ++i) us += U[i] * S[i];
+            for (int i = 0; i < SL; ++i) us += U[i] * S[i];
+            us += __shfl_xor(us, 16, WAVE);
+            us += __shfl_xor(us, 32, WAVE);
+            float acc = 0.f;
 #pragma unroll
-            for (int i = 0; i < DK; ++i) {
+            for (int i = 0; i < SL; ++i) {
                 S[i] = W[i] * S[i] - AU[i] * us + K[i] * v;
                 acc += S[i] * R[i];
             }
-        } else {
+            acc += __shfl_xor(acc, 16, WAVE);
+            acc += __shfl_xor(acc, 32, WAVE);
+            if (live && g == 0) o[(size_t)t * heads * dv + h * dv + j] = acc;
+        }
+        if (live) {
+#pragma unroll
+            for (int i = 0; i < SL; ++i) col[(size_t)i * dv] = S[i];
+        }
+    } else {
+        const int dk = dk_rt, j = blockIdx.z * 64 + threadIdx.x;
+        const bool live = j < dv;
+        const int jj = live ? j : dv - 1;
+        float *col = state + (((size_t)state_slot[r] * heads + h) * dk) * dv + jj;     // S[i][j] at col[i * dv]
+        if (fresh && live)
+            for (int i = 0; i < dk; ++i) col[(size_t)i * dv] = 0.f;
+        for (int t = t0; t < t1; ++t) {
+            const float v = to_f32(proj[(size_t)t * row_stride + off_v + h * dv + jj]);
             const float *p = prep + ((size_t)t * heads + h) * 5 * dk;
-            float us = 0.f;
+            float us = 0.f, acc = 0.f;
             for (int i = 0; i < dk; ++i) us += p[2 * dk + i] * col[(size_t)i * dv];
             for (int i = 0; i < dk; ++i) {
                 const float s = p[i] * col[(size_t)i * dv] - p[dk + i] * us + p[3 * dk + i] * v;
                 if (live) col[(size_t)i * dv] = s;
                 acc += s * p[4 * dk + i];
             }
+            if (live) o[(size_t)t * heads * dv + h * dv + j] = acc;
         }
-        if (live) o[(size_t)t * heads * dv + h * dv + j] = acc;
-    }
-    if (DK > 0 && live) {
-#pragma unroll
-        for (int i = 0; i < DK; ++i) col[(size_t)i * dv] = S[i];
     }
 }
 
@@ -156,15 +181,18 @@ static int delta_rule_t(const T *proj, int row_stride, int off_r, int off_k, int
     if (threads > 256) threads = 256;
     delta_prep_kernel<T><<<dim3(n, heads), dim3(threads), 0, stream>>>(proj, row_stride, off_r, off_k, off_a, off_l, w2, w0, a_bias, prep, heads, dk, rank);
     LCU_LAUNCH_CHECK();
-    dim3 grid(n_req, heads, (dv + 63) / 64);
-#define SCAN(DK) delta_scan_kernel<T, DK><<<grid, dim3(64), 0, stream>>>(proj, row_stride, off_v, prep, state, o, q_start, ctx_len, state_slot, heads, dk, dv)
+#define SCAN(DK) delta_scan_kernel<T, DK><<<dim3(n_req, heads, (dv + (DK ? SCAN_COLS : 64) - 1) / (DK ? SCAN_COLS : 64)), dim3(64), 0, stream>>>(proj, row_stride, off_v, prep, state, o, q_start, ctx_len, state_slot, heads, dk, dv)
     switch (dk) {
     case 16: SCAN(16); break;
     case 32: SCAN(32); break;
     case 48: SCAN(48); break;
     case 64: SCAN(64); break;
+    case 80: SCAN(80); break;
     case 96: SCAN(96); break;
+    case 112: SCAN(112); break;
     case 128: SCAN(128); break;
+    case 192: SCAN(192); break;
+    case 256: SCAN(256); break;
     default: SCAN(0); break;
     }
 #undef SCAN
@@ -183,7 +211,7 @@ LCU_API int lcu_delta_rule(const void *proj, int type, int row_stride, int off_r
                            const int *ctx_len, const int *state_slot, int n, int n_req, int heads, int dk, int dv,
                            int rank, float eps, hipStream_t stream) {
     if (n <= 0 || n_req <= 0) return LCU_OK;
-    if (heads <= 0 || heads > 65535 || dk <= 0 || dv <= 0 || rank <= 0 || rank > MAX_RANK || dv > 64 * 65535) return LCU_BAD_ARGUMENT;
+    if (heads <= 0 || heads > 65535 || dk <= 0 || dv <= 0 || rank <= 0 || rank > MAX_RANK || dv > 16 * 65535) return LCU_BAD_ARGUMENT;
     if (type == LCU_F32)
         return delta_rule_t<float>((const float *)proj, row_stride, off_r, off_k, off_v, off_g, off_a, off_l, w2, w0, a_bias, weight, prep, o, state, (float *)out, q_start, ctx_len, state_slot, n, n_req, heads, dk, dv, rank, eps, stream);
     if (type == LCU_BF16)

@@ -35,7 +35,7 @@ HOST_FLAGS = ["-O2", "-std=c++17", "-shared", "-fPIC", "-Wall", "-pthread", "-ff
 # extra flags for experiments (they enter the hash in the libraries' names)
 HIP_FLAGS += os.environ.get("LCU_HIP_FLAGS", "").split()
 
-KERNEL_LIBRARIES = ["elementwise", "rope_kv", "attention_generic", "attention_mfma", "gemm_generic", "gemm_skinny",
+KERNEL_LIBRARIES = ["elementwise", "rope_kv", "attention_generic", "attention_mfma", "attention_mfma_bias", "gemm_generic", "gemm_skinny",
                     "gemm_mid", "sampling", "random_fill", "norm_conv", "qk_norm", "delta_rule", "moe"]
 HOST_LIBRARY = "host"
 

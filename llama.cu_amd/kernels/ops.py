@@ -382,21 +382,24 @@ def mfma_attention_supported(q: torch.Tensor, n_heads: int, n_kv_heads: int, hea
 
 
 def attention_decode(q, out, cache, block_table, q_start, ctx_len, n_req, n_heads, n_kv_heads, head_dim, page_size,
-                     scale, window, n_splits, req_list: Optional[torch.Tensor] = None) -> torch.Tensor:
+                     scale, window, n_splits, req_list: Optional[torch.Tensor] = None,
+                     head_slopes: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Matrix-core attention for requests that feed one token each: all ``n_req`` requests of
-    the batch, or the ``n_req`` whose indices ``req_list`` holds."""
+    the batch, or the ``n_req`` whose indices ``req_list`` holds.  ``head_slopes``: the bias on the distance inside
+    the scores (the kernels of the second library, ``attention_mfma_bias``)."""
     if req_list is not None:
         _i32(req_list, "req_list", n_req)
     part_o = part_ml = None
     if n_splits > 1:
         part_o = torch.empty(n_req * n_heads * n_splits * head_dim, dtype=torch.float32, device=q.device)
         part_ml = torch.empty(n_req * n_heads * n_splits * 2, dtype=torch.float32, device=q.device)
-    lib = build.load("attention_mfma")
+    lib = build.load("attention_mfma" if head_slopes is None else "attention_mfma_bias")
+    more = () if head_slopes is None else (_ptr(head_slopes),)
     _check(lib.lcu_attention_decode_bf16(_ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(cache), _ptr(block_table),
                                          block_table.shape[1], _ptr(q_start), _ptr(ctx_len), _ptr(req_list), n_req, n_heads,
                                          n_kv_heads,
                                          head_dim, page_size, ctypes.c_float(scale), int(window), int(n_splits),
-                                         _ptr(part_o), _ptr(part_ml), _stream()), "attention_decode")
+                                         _ptr(part_o), _ptr(part_ml), _stream(), *more), "attention_decode")
     return out
 
 
@@ -437,7 +440,8 @@ def prefill_tasks(q_lens, ctx_lens, tokens_per_task: int, device, skip_single: b
 
 
 def attention_prefill(q, out, cache, block_table, q_start, ctx_len, task_req, task_tok0, n_tasks, tasks_per_wg, n_heads,
-                      n_kv_heads, head_dim, page_size, scale, window, n_tasks_dev: Optional[torch.Tensor] = None) -> torch.Tensor:
+                      n_kv_heads, head_dim, page_size, scale, window, n_tasks_dev: Optional[torch.Tensor] = None,
+                      head_slopes: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Matrix-core attention for any mix of portions and single tokens.  ``n_tasks_dev`` (int32 on the device, one
     entry): the lists hold that many tasks, at most ``n_tasks``, for which the grid is made."""
     if task_req.numel() < n_tasks or task_tok0.numel() < n_tasks:
@@ -446,12 +450,13 @@ def attention_prefill(q, out, cache, block_table, q_start, ctx_len, task_req, ta
     if n_tasks_dev is not None:
         _gpu(n_tasks_dev)
         _i32(n_tasks_dev, "n_tasks_dev")
-    lib = build.load("attention_mfma")
+    lib = build.load("attention_mfma" if head_slopes is None else "attention_mfma_bias")
+    more = () if head_slopes is None else (_ptr(head_slopes),)
     _check(lib.lcu_attention_prefill_bf16(_ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(cache),
                                           ctypes.c_longlong(cache.shape[0]), _ptr(block_table),
                                           block_table.shape[1], _ptr(q_start), _ptr(ctx_len), _ptr(task_req),
                                           _ptr(task_tok0), n_tasks, _ptr(n_tasks_dev), tasks_per_wg, n_heads, n_kv_heads, head_dim,
-                                          page_size, ctypes.c_float(scale), int(window), _stream()), "attention_prefill")
+                                          page_size, ctypes.c_float(scale), int(window), _stream(), *more), "attention_prefill")
     return out
 
 
@@ -550,10 +555,14 @@ def paged_attention(q: torch.Tensor, out: torch.Tensor, cache: torch.Tensor, ste
                     n_kv_heads: int, head_dim: int, page_size: int, scale: float, window: int = 0,
                     force_generic: bool = False, head_slopes: Optional[torch.Tensor] = None, value_dim: int = 0) -> torch.Tensor:
     """Attention for the batch ``step`` (an engine.batch.StepContext) over cache group
-    ``group``: picks the kernel for the batch's shape and type.  A bias inside the scores
-    (``head_slopes``) is the generic kernel's: the matrix-core kernels take none."""
+    ``group``: picks the kernel for the batch's shape and type.  With a bias inside the scores
+    (``head_slopes``) the matrix-core kernels are those of the second library, which need a positive scale."""
     bt = step.block_table(group)
-    if force_generic or head_slopes is not None or (value_dim and value_dim != head_dim) \
+    if head_slopes is not None:
+        _gpu(head_slopes)
+        if head_slopes.dtype != torch.float32 or head_slopes.shape != (n_heads,) or not head_slopes.is_contiguous():
+            raise KernelError(f"attention: head_slopes must be contiguous float32 [{n_heads}]")
+    if force_generic or (head_slopes is not None and not scale > 0) or (value_dim and value_dim != head_dim) \
             or not mfma_attention_supported(q, n_heads, n_kv_heads, head_dim, page_size):
         return paged_attention_generic(q, out, cache, bt, step.q_start, step.ctx_len, step.req_of_token, n_heads,
                                        n_kv_heads, head_dim, page_size, scale, window, head_slopes, value_dim)
@@ -564,16 +573,17 @@ def paged_attention(q: torch.Tensor, out: torch.Tensor, cache: torch.Tensor, ste
         # the workgroups start in the order of the requests' list: the requests with the most keys first, where the
         # batch says which they are (64 requests of 150 to 2,200 keys: the step 11.2 -> 11.0 ms)
         return attention_decode(q, out, cache, bt, step.q_start, step.ctx_len, step.n_req, n_heads, n_kv_heads, head_dim,
-                                page_size, scale, window, splits, req_list=step.decode_order)
+                                page_size, scale, window, splits, req_list=step.decode_order, head_slopes=head_slopes)
     # a mixed batch: the requests that decode one token go to the decode kernel, the portions
     # to the prefill kernel (each would be slow at the other's work)
     plan = plan_attention(step, n_heads, n_kv_heads, window)
     if plan.n_single:
         attention_decode(q, out, cache, bt, step.q_start, step.ctx_len, plan.n_single, n_heads, n_kv_heads, head_dim, page_size,
-                         scale, window, plan.single_splits, req_list=plan.singles)
+                         scale, window, plan.single_splits, req_list=plan.singles, head_slopes=head_slopes)
     if plan.max_tasks:
         attention_prefill(q, out, cache, bt, step.q_start, step.ctx_len, plan.task_req, plan.task_tok0, plan.max_tasks,
-                          plan.per_wg, n_heads, n_kv_heads, head_dim, page_size, scale, window, n_tasks_dev=plan.n_tasks_dev)
+                          plan.per_wg, n_heads, n_kv_heads, head_dim, page_size, scale, window, n_tasks_dev=plan.n_tasks_dev,
+                          head_slopes=head_slopes)
     return out
 
 

@@ -105,8 +105,8 @@ class Attention(Part):
             # a bfloat16 model whose attention the matrix-core kernels do not take still runs, on the generic
             # kernel: correct, and several times slower over long contexts, so the log says so and why
             why = ops.mfma_attention_refusal(self.dtype, self.heads, self.kv_heads, self.head_dim, self.own_page_size or self.page_size)
-            if why is None and self.position.score_slopes() is not None:
-                why = "the position encoding is a bias inside the scores, which the matrix-core kernels do not take"
+            if why is None and self.position.score_slopes() is not None and not self.scale > 0:
+                why = "with a bias inside the scores the matrix-core kernels need a positive scale"
             if why is None and self.value_dim != self.head_dim:
                 why = f"the values' head size {self.value_dim} is not the keys' {self.head_dim}"
             if why is not None:
@@ -118,8 +118,8 @@ class Attention(Part):
         the host, and go to the device with the step's arrays; ``forward`` then launches work whose sizes follow from
         the step's sizes alone."""
         page_size = self.own_page_size or self.page_size
-        if self.dtype == torch.bfloat16 and self.position.score_slopes() is None and self.value_dim == self.head_dim \
-                and ops.mfma_attention_refusal(self.dtype, self.heads, self.kv_heads, self.head_dim, page_size) is None:
+        if self.dtype == torch.bfloat16 and (self.position.score_slopes() is None or self.scale > 0) \
+                and self.value_dim == self.head_dim and ops.mfma_attention_refusal(self.dtype, self.heads, self.kv_heads, self.head_dim, page_size) is None:
             ops.plan_attention(step, self.heads, self.kv_heads, self.window)
 
     # forward(..., into=(residual, norm)) may end with the residual sum and that norm's weight
