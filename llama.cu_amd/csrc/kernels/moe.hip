@@ -2,8 +2,8 @@
 //
 //   route:   z = W_router h (32-bit), the `top` experts with the largest z (ties: the lower
 //            index), each with the weight sigmoid(z) (not renormalised);
-//   group:   the (token, choice) pairs sorted by expert and cut into tiles of 64 rows of one
-//            expert, on the device (nothing comes back to the host);
+//   group:   the (token, choice) pairs sorted by expert and cut into tiles of up to 16 or 64 rows of
+//            one expert, on the device (nothing comes back to the host);
 //   up:      act = gelu(W_up[e] (weight * h))    the weight multiplies the expert's INPUT
 //   down:    y = W_down[e] act, added to the token's output row (32-bit).
 // The products run on the matrix cores: bfloat16 operands with v_mfma_f32_16x16x32_bf16, or
@@ -13,7 +13,7 @@
 #include "common.h"
 
 constexpr int MOE_MAX_EXPERTS = 1024;
-constexpr int MOE_TILE_ROWS = 64;
+constexpr int MOE_TILE_ROWS = 64;        // rows of a tile of the kernel for many rows; the kernel for few rows takes 16
 
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
@@ -21,7 +21,11 @@ typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 
 // ---------------------------------------------------------------- route
 // One block of 256 threads per token.  h: [n, d] of T; router: [experts, d] 32-bit.
-// ids, wts: [n, top].
+// ids, wts: [n, top].  A wave takes the experts e = wave, wave + 4, ...; with d a multiple of 8 a lane
+// keeps its share of the row (eight neighbouring elements of every 512) in registers for all of them.
+template <class T> struct alignas(8 * sizeof(T)) Row8 { T v[8]; };
+constexpr int ROUTE_CHUNKS = 8;                  // rows of up to 8 * 512 elements stay in registers
+
 template <class T>
 __global__ void __launch_bounds__(256)
 moe_route_kernel(const T *__restrict__ h, const float *__restrict__ router, int *__restrict__ ids,
@@ -29,34 +33,64 @@ moe_route_kernel(const T *__restrict__ h, const float *__restrict__ router, int 
     __shared__ float z[MOE_MAX_EXPERTS];
     const int t = blockIdx.x, wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
     const T *row = h + (size_t)t * d;
-    for (int e = wave; e < experts; e += 256 / WAVE) {
-        const float *w = router + (size_t)e * d;
-        float acc = 0.f;
-        for (int c = lane; c < d; c += WAVE) acc += to_f32(row[c]) * w[c];
-        acc = wave_sum(acc);
-        if (lane == 0) z[e] = acc;
+    if (d % 8 == 0 && d <= ROUTE_CHUNKS * 512) {
+        float x[ROUTE_CHUNKS][8];
+#pragma unroll
+        for (int k = 0; k < ROUTE_CHUNKS; ++k) {
+            const int c = k * 512 + lane * 8;
+            if (c < d) {
+                const Row8<T> in = *(const Row8<T> *)(row + c);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) x[k][e] = to_f32(in.v[e]);
+            }
+        }
+        for (int e = wave; e < experts; e += 256 / WAVE) {
+            const float *w = router + (size_t)e * d;
+            float acc = 0.f;
+#pragma unroll
+            for (int k = 0; k < ROUTE_CHUNKS; ++k) {
+                const int c = k * 512 + lane * 8;
+                if (c < d) {
+                    const f32x4 w0 = *(const f32x4 *)(w + c), w1 = *(const f32x4 *)(w + c + 4);
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) acc += x[k][i] * w0[i];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) acc += x[k][4 + i] * w1[i];
+                }
+            }
+            acc = wave_sum(acc);
+            if (lane == 0) z[e] = acc;
+        }
+    } else {
+        for (int e = wave; e < experts; e += 256 / WAVE) {
+            const float *w = router + (size_t)e * d;
+            float acc = 0.f;
+            for (int c = lane; c < d; c += WAVE) acc += to_f32(row[c]) * w[c];
+            acc = wave_sum(acc);
+            if (lane == 0) z[e] = acc;
+        }
     }
     __syncthreads();
     for (int k = 0; k < top; ++k) {                  // the first wave chooses; the others only keep the barriers
         if (wave == 0) {
-        float best = -INFINITY;
-        int arg = 0x7fffffff;
-        for (int e = lane; e < experts; e += WAVE) {
-            const float v = z[e];
-            if (v > best || (v == best && e < arg)) { best = v; arg = e; }
-        }
+            float best = -INFINITY;
+            int arg = 0x7fffffff;
+            for (int e = lane; e < experts; e += WAVE) {
+                const float v = z[e];
+                if (v > best || (v == best && e < arg)) { best = v; arg = e; }
+            }
 #pragma unroll
-        for (int off = 32; off > 0; off >>= 1) {
-            const float ob = __shfl_xor(best, off, WAVE);
-            const int oa = __shfl_xor(arg, off, WAVE);
-            if (ob > best || (ob == best && oa < arg)) { best = ob; arg = oa; }
-        }
-        if (arg >= experts) arg = 0;                 // every logit NaN: any expert
-        if (lane == 0) {
-            ids[(size_t)t * top + k] = arg;
-            wts[(size_t)t * top + k] = 1.0f / (1.0f + expf(-z[arg]));
-            z[arg] = -INFINITY;
-        }
+            for (int off = 32; off > 0; off >>= 1) {
+                const float ob = __shfl_xor(best, off, WAVE);
+                const int oa = __shfl_xor(arg, off, WAVE);
+                if (ob > best || (ob == best && oa < arg)) { best = ob; arg = oa; }
+            }
+            if (arg >= experts) arg = 0;                 // every logit NaN: any expert
+            if (lane == 0) {
+                ids[(size_t)t * top + k] = arg;
+                wts[(size_t)t * top + k] = 1.0f / (1.0f + expf(-z[arg]));
+                z[arg] = -INFINITY;
+            }
         }
         __syncthreads();
     }
@@ -64,12 +98,12 @@ moe_route_kernel(const T *__restrict__ h, const float *__restrict__ router, int 
 
 // ---------------------------------------------------------------- group
 // One block.  ids: [total] experts of the (token, choice) pairs in flat order.  Writes
-// sorted_to_flat [total] (the pairs sorted by expert), and the tiles: tile_expert, tile_begin
-// (first sorted row), tile_rows, each [max_tiles], and n_tiles [1].
+// sorted_to_flat [total] (the pairs sorted by expert), and the tiles of up to rows_per_tile rows:
+// tile_expert, tile_begin (first sorted row), tile_rows, each [max_tiles], and n_tiles [1].
 __global__ void __launch_bounds__(1024)
 moe_group_kernel(const int *__restrict__ ids, int total, int experts, int *__restrict__ sorted_to_flat,
                  int *__restrict__ tile_expert, int *__restrict__ tile_begin, int *__restrict__ tile_rows,
-                 int *__restrict__ n_tiles, int max_tiles) {
+                 int *__restrict__ n_tiles, int max_tiles, int rows_per_tile) {
     __shared__ int count[MOE_MAX_EXPERTS];
     __shared__ int cursor[MOE_MAX_EXPERTS];
     for (int e = threadIdx.x; e < experts; e += blockDim.x) count[e] = 0;
@@ -80,10 +114,10 @@ moe_group_kernel(const int *__restrict__ ids, int total, int experts, int *__res
         int at = 0, tiles = 0;
         for (int e = 0; e < experts; ++e) {
             cursor[e] = at;
-            for (int r = 0; r < count[e] && tiles < max_tiles; r += MOE_TILE_ROWS) {
+            for (int r = 0; r < count[e] && tiles < max_tiles; r += rows_per_tile) {
                 tile_expert[tiles] = e;
                 tile_begin[tiles] = at + r;
-                tile_rows[tiles] = count[e] - r < MOE_TILE_ROWS ? count[e] - r : MOE_TILE_ROWS;
+                tile_rows[tiles] = count[e] - r < rows_per_tile ? count[e] - r : rows_per_tile;
                 ++tiles;
             }
             at += count[e];
@@ -133,22 +167,42 @@ __device__ __forceinline__ float gelu_erf(float z) { return 0.5f * z * (1.0f + e
 
 enum { MOE_UP = 0, MOE_DOWN = 1 };
 
-// A block of four waves takes one tile (up to 64 sorted rows of one expert) and 64 output
-// features, a wave 16 of the features for all rows.  The weight is the instruction's first
-// operand (16 features x k), the rows the second (k x 16 rows): a lane then holds four
-// neighbouring features of one row.
-//   MOE_UP:   x = h [n, K], row = token of the pair, scaled by the pair's weight; out_t = act
+// Both kernels below multiply the rows of a tile (sorted rows of one expert) with that expert's matrix
+// w[e] ([N, K], row-major) on the matrix cores.  The weight is the instruction's first operand (16
+// features x k), the rows the second (k x 16 rows): a lane then holds four neighbouring features of
+// one row.  Rows and features beyond the tile's or the matrix's end are computed from clamped
+// addresses and never stored.  K is a multiple of the elements in 16 bytes.
+//   MOE_UP:   x = h [n, K], a row is the token of its pair, scaled by the pair's weight; out_t = act
 //             [total, N] at the sorted row, gelu applied.
 //   MOE_DOWN: x = act [total, K] at the sorted row; out_f [total or n, N] 32-bit at the flat pair
 //             (add == 0: stored) or at the pair's token (add == 1: added; only with top == 1).
 template <class T, int MODE>
+__device__ __forceinline__ void moe_store(const f32x4 &acc, int dst, int col0, int N, T *__restrict__ out_t,
+                                          float *__restrict__ out_f, int out_stride, int add) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int col = col0 + i;
+        if (col >= N) continue;
+        if (MODE == MOE_UP) {
+            out_t[(size_t)dst * out_stride + col] = from_f32<T>(gelu_erf(acc[i]));
+        } else {
+            float *o = out_f + (size_t)dst * out_stride + col;
+            *o = add ? *o + acc[i] : acc[i];
+        }
+    }
+}
+
+// Few rows an expert (decoding): tiles of up to 16 rows; a block of four waves takes a tile and 64
+// features, a wave 16 of them, and streams its 16 rows of the weight once, four steps of loads in flight.
+template <class T, int MODE>
 __global__ void __launch_bounds__(256)
-moe_gemm_kernel(const T *__restrict__ x, int x_stride, const T *__restrict__ w, size_t w_expert_stride, int N, int K,
-                const int *__restrict__ sorted_to_flat, const float *__restrict__ wts,
-                const int *__restrict__ tile_expert, const int *__restrict__ tile_begin,
-                const int *__restrict__ tile_rows, const int *__restrict__ n_tiles, T *__restrict__ out_t,
-                float *__restrict__ out_f, int out_stride, int top, int add) {
+moe_gemm_few_kernel(const T *__restrict__ x, int x_stride, const T *__restrict__ w, size_t w_expert_stride, int N, int K,
+                    const int *__restrict__ sorted_to_flat, const float *__restrict__ wts,
+                    const int *__restrict__ tile_expert, const int *__restrict__ tile_begin,
+                    const int *__restrict__ tile_rows, const int *__restrict__ n_tiles, T *__restrict__ out_t,
+                    float *__restrict__ out_f, int out_stride, int top, int add) {
     typedef Mma<T> M;
+    typedef typename M::frag frag;
     const int tile = blockIdx.x;
     if (tile >= n_tiles[0]) return;
     const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE, g = lane / 16, l16 = lane % 16;
@@ -156,57 +210,133 @@ moe_gemm_kernel(const T *__restrict__ x, int x_stride, const T *__restrict__ w, 
     if (f0 >= N) return;
     const int e = tile_expert[tile], row0 = tile_begin[tile], rows = tile_rows[tile];
     const int f = f0 + l16;
-    const T *wrow = w + (size_t)e * w_expert_stride + (size_t)(f < N ? f : N - 1) * K;
-    const T *xrow[4];
-    float sc[4];
-    int dst[4];
-    bool valid[4];
+    const T *wrow = w + (size_t)e * w_expert_stride + (size_t)(f < N ? f : N - 1) * K + g * M::PER_LANE;
+    const bool valid = l16 < rows;
+    const int srow = row0 + (valid ? l16 : 0);
+    const int flat = sorted_to_flat[srow];
+    const T *xrow = (MODE == MOE_UP ? x + (size_t)(flat / top) * x_stride : x + (size_t)srow * x_stride) + g * M::PER_LANE;
+    const float sc = MODE == MOE_UP ? wts[flat] : 1.f;
+    const int dst = MODE == MOE_UP ? srow : (add ? flat / top : flat);
+    f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+    const int kfull = K / M::KSTEP * M::KSTEP;
+    int k0 = 0;
+    for (; k0 + 4 * M::KSTEP <= kfull; k0 += 4 * M::KSTEP) {
+        frag a[4], b[4];
 #pragma unroll
-    for (int m = 0; m < 4; ++m) {
-        valid[m] = 16 * m + l16 < rows;
-        const int srow = row0 + (valid[m] ? 16 * m + l16 : 0);
-        const int flat = sorted_to_flat[srow];
-        sc[m] = 1.f;
-        if (MODE == MOE_UP) {
-            xrow[m] = x + (size_t)(flat / top) * x_stride;
-            sc[m] = wts[flat];
-            dst[m] = srow;
-        } else {
-            xrow[m] = x + (size_t)srow * x_stride;
-            dst[m] = add ? flat / top : flat;
-        }
+        for (int u = 0; u < 4; ++u) a[u] = __builtin_nontemporal_load((const frag *)(wrow + k0 + u * M::KSTEP));
+#pragma unroll
+        for (int u = 0; u < 4; ++u) b[u] = M::load(xrow + k0 + u * M::KSTEP);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) acc = M::mma(a[u], MODE == MOE_UP ? M::scaled(b[u], sc) : b[u], acc);
     }
-    f32x4 acc[4];
-#pragma unroll
-    for (int m = 0; m < 4; ++m) acc[m] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (; k0 < K; k0 += M::KSTEP) {                 // the steps that are left, the last one perhaps in part
+        const bool in = k0 + g * M::PER_LANE < K;
+        const frag a = in ? M::load(wrow + k0) : M::zero();
+        const frag b = in ? M::load(xrow + k0) : M::zero();
+        acc = M::mma(a, MODE == MOE_UP ? M::scaled(b, sc) : b, acc);
+    }
+    if (valid) moe_store<T, MODE>(acc, dst, f0 + 4 * g, N, out_t, out_f, out_stride, add);
+}
 
-    for (int k0 = 0; k0 < K; k0 += M::KSTEP) {
-        const int kk = k0 + g * M::PER_LANE;
-        const bool in = kk < K;
-        const typename M::frag a = (in && f < N) ? M::load(wrow + kk) : M::zero();
+// Many rows an expert (prompts): tiles of up to 64 rows; a block of four waves takes a tile and 128
+// features.  Rows and weights go through LDS in steps of 128 bytes of k, the next step's loads on their
+// way while one is multiplied; a wave multiplies 32 features with all 64 rows (eight sums).
+template <class T, int MODE>
+__global__ void __launch_bounds__(256)
+moe_gemm_many_kernel(const T *__restrict__ x, int x_stride, const T *__restrict__ w, size_t w_expert_stride, int N, int K,
+                     const int *__restrict__ sorted_to_flat, const float *__restrict__ wts,
+                     const int *__restrict__ tile_expert, const int *__restrict__ tile_begin,
+                     const int *__restrict__ tile_rows, const int *__restrict__ n_tiles, T *__restrict__ out_t,
+                     float *__restrict__ out_f, int out_stride, int top, int add) {
+    typedef Mma<T> M;
+    typedef typename M::frag frag;
+    constexpr int PL = M::PER_LANE;                 // elements in 16 bytes
+    constexpr int KS = 128 / sizeof(T);             // elements of k a step
+    constexpr int CH = KS / PL;                     // 16-byte pieces of a row a step: 8
+    constexpr int LD = KS + PL;                     // a row in LDS, with a piece of padding against bank conflicts
+    __shared__ __attribute__((aligned(16))) T xs[64 * LD];
+    __shared__ __attribute__((aligned(16))) T ws[128 * LD];
+    const int tile = blockIdx.x;
+    if (tile >= n_tiles[0]) return;
+    const int n0 = blockIdx.y * 128;
+    const int e = tile_expert[tile], row0 = tile_begin[tile], rows = tile_rows[tile];
+    const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE, g = lane / 16, l16 = lane % 16;
+    const int ch = tid % CH;                        // this thread's piece of k in every row it copies
+    const T *xptr[2];
+    float xsc[2];
 #pragma unroll
-        for (int m = 0; m < 4; ++m) {
-            if (16 * m < rows) {
-                typename M::frag b = (in && valid[m]) ? M::load(xrow[m] + kk) : M::zero();
-                if (MODE == MOE_UP) b = M::scaled(b, sc[m]);
-                acc[m] = M::mma(a, b, acc[m]);
+    for (int i = 0; i < 2; ++i) {
+        const int r = tid / CH + 32 * i;
+        const int srow = row0 + (r < rows ? r : 0);
+        if (MODE == MOE_UP) {
+            const int flat = sorted_to_flat[srow];
+            xptr[i] = x + (size_t)(flat / top) * x_stride + ch * PL;
+            xsc[i] = wts[flat];
+        } else {
+            xptr[i] = x + (size_t)srow * x_stride + ch * PL;
+            xsc[i] = 1.f;
+        }
+    }
+    const T *wptr[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int fr = n0 + tid / CH + 32 * i;
+        wptr[i] = w + (size_t)e * w_expert_stride + (size_t)(fr < N ? fr : N - 1) * K + ch * PL;
+    }
+    frag xreg[2], wreg[4];
+    auto from_memory = [&](int k0) {
+        const bool in = k0 + ch * PL < K;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) wreg[i] = in ? M::load(wptr[i] + k0) : M::zero();
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            xreg[i] = in ? M::load(xptr[i] + k0) : M::zero();
+            if (MODE == MOE_UP) xreg[i] = M::scaled(xreg[i], xsc[i]);
+        }
+    };
+    f32x4 acc[2][4];
+#pragma unroll
+    for (int ft = 0; ft < 2; ++ft)
+#pragma unroll
+        for (int m = 0; m < 4; ++m) acc[ft][m] = f32x4{0.f, 0.f, 0.f, 0.f};
+    from_memory(0);
+    for (int k0 = 0; k0 < K; k0 += KS) {
+        __syncthreads();                            // the step before has been read
+#pragma unroll
+        for (int i = 0; i < 2; ++i) *(frag *)(xs + (tid / CH + 32 * i) * LD + ch * PL) = xreg[i];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) *(frag *)(ws + (tid / CH + 32 * i) * LD + ch * PL) = wreg[i];
+        __syncthreads();
+        if (k0 + KS < K) from_memory(k0 + KS);
+#pragma unroll
+        for (int ks = 0; ks < KS / M::KSTEP; ++ks) {
+            frag a[2], b[4];
+#pragma unroll
+            for (int ft = 0; ft < 2; ++ft) a[ft] = *(const frag *)(ws + (32 * wave + 16 * ft + l16) * LD + ks * M::KSTEP + g * PL);
+#pragma unroll
+            for (int m = 0; m < 4; ++m) b[m] = *(const frag *)(xs + (16 * m + l16) * LD + ks * M::KSTEP + g * PL);
+#pragma unroll
+            for (int m = 0; m < 4; ++m) {
+                if (16 * m < rows) {
+#pragma unroll
+                    for (int ft = 0; ft < 2; ++ft) acc[ft][m] = M::mma(a[ft], b[m], acc[ft][m]);
+                }
             }
         }
     }
 #pragma unroll
     for (int m = 0; m < 4; ++m) {
-        if (!valid[m]) continue;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int col = f0 + 4 * g + i;
-            if (col >= N) continue;
-            if (MODE == MOE_UP) {
-                out_t[(size_t)dst[m] * out_stride + col] = from_f32<T>(gelu_erf(acc[m][i]));
-            } else {
-                float *o = out_f + (size_t)dst[m] * out_stride + col;
-                *o = add ? *o + acc[m][i] : acc[m][i];
-            }
+        const int r = 16 * m + l16;
+        if (r >= rows) continue;
+        const int srow = row0 + r;
+        int dst = srow;
+        if (MODE == MOE_DOWN) {
+            const int flat = sorted_to_flat[srow];
+            dst = add ? flat / top : flat;
         }
+#pragma unroll
+        for (int ft = 0; ft < 2; ++ft)
+            moe_store<T, MODE>(acc[ft][m], dst, n0 + 32 * wave + 16 * ft + 4 * g, N, out_t, out_f, out_stride, add);
     }
 }
 
@@ -221,7 +351,9 @@ __global__ void moe_combine_kernel(float *__restrict__ out, const float *__restr
     }
 }
 
-LCU_API int lcu_moe_tile_rows() { return MOE_TILE_ROWS; }
+// Rows of a tile for n * top pairs over so many experts: 16 (the kernel for few rows) while an expert has 16 rows
+// or fewer on average, else 64.  The caller sizes its scratch with it: max_tiles = min(total, total / rows + experts).
+LCU_API int lcu_moe_tile_rows(int total, int experts) { return (long long)total <= 16ll * experts ? 16 : MOE_TILE_ROWS; }
 
 // h: [n, d] of `type`; router: [experts, d] 32-bit; ids, wts: [n * top].
 LCU_API int lcu_moe_route(const void *h, int type, const float *router, int *ids, float *wts, int n, int d, int experts,
@@ -248,19 +380,25 @@ LCU_API int lcu_moe_experts(const void *h, int type, const int *ids, const float
         (type != LCU_F32 && type != LCU_BF16))
         return LCU_BAD_ARGUMENT;
     const int total = n * top;
+    const int tile_rows = lcu_moe_tile_rows(total, experts);
     int *sorted = ints, *t_exp = ints + total, *t_beg = t_exp + max_tiles, *t_rows = t_beg + max_tiles, *n_tiles = t_rows + max_tiles;
-    moe_group_kernel<<<dim3(1), dim3(1024), 0, stream>>>(ids, total, experts, sorted, t_exp, t_beg, t_rows, n_tiles, max_tiles);
+    moe_group_kernel<<<dim3(1), dim3(1024), 0, stream>>>(ids, total, experts, sorted, t_exp, t_beg, t_rows, n_tiles, max_tiles, tile_rows);
     LCU_LAUNCH_CHECK();
     const int add = top == 1;
     float *down_to = add ? out : y;
-    dim3 block(256), gu(max_tiles, (ff + 63) / 64), gd(max_tiles, (d + 63) / 64);
+    const int per_block = tile_rows == 16 ? 64 : 128;         // features a block takes
+    dim3 block(256), gu(max_tiles, (ff + per_block - 1) / per_block), gd(max_tiles, (d + per_block - 1) / per_block);
+#define GO(KERNEL, T)                                                                                                              \
+    KERNEL<T, MOE_UP><<<gu, block, 0, stream>>>((const T *)h, d, (const T *)w_up, (size_t)ff * d, ff, d, sorted, wts, t_exp, t_beg, \
+                                                t_rows, n_tiles, (T *)act, nullptr, ff, top, 0);                                    \
+    KERNEL<T, MOE_DOWN><<<gd, block, 0, stream>>>((const T *)act, ff, (const T *)w_down, (size_t)ff * d, d, ff, sorted, wts, t_exp, \
+                                                  t_beg, t_rows, n_tiles, nullptr, down_to, d, top, add)
     if (type == LCU_BF16) {
-        moe_gemm_kernel<bf16_t, MOE_UP><<<gu, block, 0, stream>>>((const bf16_t *)h, d, (const bf16_t *)w_up, (size_t)ff * d, ff, d, sorted, wts, t_exp, t_beg, t_rows, n_tiles, (bf16_t *)act, nullptr, ff, top, 0);
-        moe_gemm_kernel<bf16_t, MOE_DOWN><<<gd, block, 0, stream>>>((const bf16_t *)act, ff, (const bf16_t *)w_down, (size_t)ff * d, d, ff, sorted, wts, t_exp, t_beg, t_rows, n_tiles, nullptr, down_to, d, top, add);
+        if (tile_rows == 16) { GO(moe_gemm_few_kernel, bf16_t); } else { GO(moe_gemm_many_kernel, bf16_t); }
     } else {
-        moe_gemm_kernel<float, MOE_UP><<<gu, block, 0, stream>>>((const float *)h, d, (const float *)w_up, (size_t)ff * d, ff, d, sorted, wts, t_exp, t_beg, t_rows, n_tiles, (float *)act, nullptr, ff, top, 0);
-        moe_gemm_kernel<float, MOE_DOWN><<<gd, block, 0, stream>>>((const float *)act, ff, (const float *)w_down, (size_t)ff * d, d, ff, sorted, wts, t_exp, t_beg, t_rows, n_tiles, nullptr, down_to, d, top, add);
+        if (tile_rows == 16) { GO(moe_gemm_few_kernel, float); } else { GO(moe_gemm_many_kernel, float); }
     }
+#undef GO
     LCU_LAUNCH_CHECK();
     if (!add) {
         moe_combine_kernel<<<dim3((d + 255) / 256, n < 65535 ? n : 65535), dim3(256), 0, stream>>>(out, y, n, d, top);

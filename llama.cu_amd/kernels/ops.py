@@ -1152,8 +1152,8 @@ def moe_experts(h: torch.Tensor, ids: torch.Tensor, wts: torch.Tensor, w_up: tor
     if d % per or ff % per:
         raise KernelError(f"moe_experts: the width {d} and the experts' {ff} must be multiples of {per}")
     lib = build.load("moe")
-    tile = lib.lcu_moe_tile_rows()
     total = n * top
+    tile = lib.lcu_moe_tile_rows(total, experts)
     max_tiles = min(total, total // tile + experts)
     ints = torch.empty(total + 3 * max_tiles + 1, dtype=torch.int32, device=h.device)
     act = torch.empty((total, ff), dtype=h.dtype, device=h.device)

@@ -161,7 +161,7 @@ def test_delta_rule_against_the_recurrence_in_any_cut(dtype, heads, dim, rank):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("experts,top,ff,n", [(5, 2, 40, 33), (12, 1, 24, 150), (3, 3, 16, 1), (9, 4, 72, 70)])
+@pytest.mark.parametrize("experts,top,ff,n", [(5, 2, 40, 33), (12, 1, 24, 150), (3, 3, 16, 1), (9, 4, 72, 70), (4, 2, 136, 300), (3, 1, 200, 260)])
 def test_mixture_of_experts(dtype, experts, top, ff, n):
     from llama_cu_amd.kernels import ops
     d, tdt = 72, TYPES[dtype]
