@@ -23,10 +23,11 @@ constexpr float DECAY_SCALE = 0.6065306597126334f;      // exp(-1/2)
 __device__ __forceinline__ float sigmoidf_(float z) { return 1.0f / (1.0f + expf(-z)); }
 
 // proj: [n, row_stride] rows that hold r, k, a_lin (dk per head each) and the low-rank
-// projection l (rank) at the given column offsets.  prep: [n, heads, 5, dk] 32-bit.
+// projection l (rank) at the given column offsets.  w2t: [rank, heads * dk], the decay's second matrix
+// transposed.  prep: [n, heads, 5, dk] 32-bit.
 template <class T>
 __global__ void delta_prep_kernel(const T *__restrict__ proj, int row_stride, int off_r, int off_k, int off_a, int off_l,
-                                  const float *__restrict__ w2, const float *__restrict__ w0,
+                                  const float *__restrict__ w2t, const float *__restrict__ w0,
                                   const float *__restrict__ a_bias, float *__restrict__ prep, int heads, int dk, int rank) {
     __shared__ float th[MAX_RANK];
     __shared__ float scratch[16];
@@ -44,7 +45,7 @@ __global__ void delta_prep_kernel(const T *__restrict__ proj, int row_stride, in
     for (int i = threadIdx.x; i < dk; i += blockDim.x) {
         const int c = h * dk + i;
         float z = w0[c];
-        for (int j = 0; j < rank; ++j) z += w2[(size_t)c * rank + j] * th[j];
+        for (int j = 0; j < rank; ++j) z += w2t[(size_t)j * heads * dk + c] * th[j];      // (neighbouring lanes, neighbouring addresses)
         const float w = expf(-DECAY_SCALE * sigmoidf_(z));
         const float a = sigmoidf_(to_f32(row[off_a + c]) + a_bias[c]);
         const float kk = to_f32(row[off_k + c]);
@@ -57,14 +58,31 @@ __global__ void delta_prep_kernel(const T *__restrict__ proj, int row_stride, in
     }
 }
 
-// DK > 0 (a multiple of 16): one wave per (request, head, 16 value channels).  The wave's lanes are four groups of 16:
-// lane (g, j) keeps the quarter g of column j of S (key channels g * DK/4 .. + DK/4 - 1) in registers, so a token
-// costs a lane DK/4 of each pass, and the two sums over key channels (u^T S and S^T r) cross the groups with two
-// shuffles each.  The token's five vectors go through LDS (all lanes copy, each reads its quarter), the next
-// token's are on their way meanwhile.
+// DK > 0 (a multiple of 16): one wave per (request, head, 16 or 8 value channels).  The wave's lanes are four groups of
+// 16 (eight of 8 where DK is a multiple of 32): lane (g, j) keeps the part g of column j of S (key channels
+// g * DK/groups .. + DK/groups - 1) in registers, so a token costs a lane DK/groups of each pass, and the two sums over
+// key channels (u^T S and S^T r) cross the groups in the vector unit.  A request's tokens are one chain, so what a
+// token costs a wave is what counts: more lanes a column make it shorter.  The tokens' five vectors go through LDS, eight tokens at a time (all lanes copy, each reads its
+// quarter), the next eight tokens' are on their way meanwhile.
 // DK == 0: any dk, one wave per (request, head, 64 value channels), the column stays in the state's memory.
 // state: [slots, heads, dk, dv]; o: [n, heads * dv] 32-bit.
-constexpr int SCAN_GROUPS = 4, SCAN_COLS = WAVE / SCAN_GROUPS;
+
+// The sum of the values that the lanes l, l + 16, l + 32 and l + 48 hold (and l + 8 of each, with eight groups), in all
+// of them, always added in the same order.  The rows of 16 lanes are swapped in the vector unit (v_permlane16_swap,
+// v_permlane32_swap): a shuffle through LDS takes far longer, and the recurrence waits for this value twice a token.
+template <int GROUPS>
+__device__ __forceinline__ float sum_over_groups(float x) {
+    if (GROUPS == 8)            // eight groups of 8 lanes: first the two groups of a row of 16 (the row rotated by 8, in the vector unit too)
+        x += __uint_as_float((unsigned)__builtin_amdgcn_update_dpp(0, (int)__float_as_uint(x), 0x128, 0xf, 0xf, false));
+    const unsigned u = __float_as_uint(x);
+    const auto a = __builtin_amdgcn_permlane16_swap(u, u, false, false);     // (rows 0 0 2 2, rows 1 1 3 3)
+    const unsigned v = __float_as_uint(__uint_as_float(a[0]) + __uint_as_float(a[1]));
+    const auto b = __builtin_amdgcn_permlane32_swap(v, v, false, false);     // (lower half twice, upper half twice)
+    return __uint_as_float(b[0]) + __uint_as_float(b[1]);
+}
+
+template <class T, int DK>
+constexpr int scan_groups() { return DK > 0 && DK % 32 == 0 ? 8 : 4; }
 
 template <class T, int DK>
 __global__ void __launch_bounds__(64)
@@ -75,59 +93,72 @@ delta_scan_kernel(const T *__restrict__ proj, int row_stride, int off_v, const f
     const int t0 = q_start[r], t1 = q_start[r + 1];
     const bool fresh = ctx_len[r] - (t1 - t0) == 0;          // the request's first token: the state starts at zero
     if constexpr (DK > 0) {
+        constexpr int SCAN_GROUPS = scan_groups<T, DK>(), SCAN_COLS = WAVE / SCAN_GROUPS;
         constexpr int SL = DK / SCAN_GROUPS;                  // key channels of a lane
         constexpr int PER_LANE = (5 * DK + 63) / 64;
+        constexpr int TB = DK <= 128 ? 8 : 4;                 // tokens whose vectors are brought in together
         const int g = threadIdx.x / SCAN_COLS, j = blockIdx.z * SCAN_COLS + threadIdx.x % SCAN_COLS;
         const bool live = j < dv;
         const int jj = live ? j : dv - 1;                     // lanes beyond dv compute along and store nothing
         float *col = state + (((size_t)state_slot[r] * heads + h) * DK + g * SL) * dv + jj;   // S[g * SL + i][j] at col[i * dv]
-        __shared__ __attribute__((aligned(16))) float vec[2][5 * DK];
+        // a vector in LDS: the four groups' quarters, each followed by four floats of padding, so that the groups' reads of
+        // their quarters (the same offset in each) fall into different banks
+        constexpr int SLP = SL + 4, VEC = SCAN_GROUPS * SLP;
+        __shared__ __attribute__((aligned(16))) float vec[2][TB][5 * VEC];
         float S[SL];
 #pragma unroll
         for (int i = 0; i < SL; ++i) S[i] = fresh ? 0.f : col[(size_t)i * dv];
-        float next[PER_LANE];
+        // the vectors and values of the next TB tokens, on their way while the TB before them are folded in: a
+        // token's own arithmetic is far shorter than a trip to memory
+        float next[TB][PER_LANE], v_next[TB];
+        const T *vp = proj + off_v + h * dv + jj;
         auto fetch = [&](int t) {
-            const float *p = prep + ((size_t)t * heads + h) * 5 * DK;
 #pragma unroll
-            for (int e = 0; e < PER_LANE; ++e) {
-                const int idx = e * 64 + threadIdx.x;
-                next[e] = idx < 5 * DK ? p[idx] : 0.f;
+            for (int b = 0; b < TB; ++b) {
+                const int tt = t + b < t1 ? t + b : t1 - 1;
+                const float *p = prep + ((size_t)tt * heads + h) * 5 * DK;
+#pragma unroll
+                for (int e = 0; e < PER_LANE; ++e) {
+                    const int idx = e * 64 + threadIdx.x;
+                    next[b][e] = idx < 5 * DK ? p[idx] : 0.f;
+                }
+                v_next[b] = to_f32(vp[(size_t)tt * row_stride]);
             }
         };
-        const T *vp = proj + off_v + h * dv + jj;
-        float v_next = 0.f;
-        if (t0 < t1) {
-            fetch(t0);
-            v_next = to_f32(vp[(size_t)t0 * row_stride]);
-        }
-        for (int t = t0; t < t1; ++t) {
-            float *cur = vec[(t - t0) & 1];
+        if (t0 < t1) fetch(t0);
+        int turn = 0;
+        for (int t = t0; t < t1; t += TB, turn ^= 1) {
+            float v[TB];
 #pragma unroll
-            for (int e = 0; e < PER_LANE; ++e) {
-                const int idx = e * 64 + threadIdx.x;
-                if (idx < 5 * DK) cur[idx] = next[e];
-            }
-            const float v = v_next;
-            __syncthreads();
-            if (t + 1 < t1) {
-                fetch(t + 1);
-                v_next = to_f32(vp[(size_t)(t + 1) * row_stride]);
-            }
-            const float *W = cur + g * SL, *AU = W + DK, *U = W + 2 * DK, *K = W + 3 * DK, *R = W + 4 * DK;
-            float us = 0.f;
+            for (int b = 0; b < TB; ++b) {
+                v[b] = v_next[b];
 #pragma unroll
-            for (int i = 0; i < SL; ++i) us += U[i] * S[i];
-            us += __shfl_xor(us, 16, WAVE);
-            us += __shfl_xor(us, 32, WAVE);
-            float acc = 0.f;
-#pragma unroll
-            for (int i = 0; i < SL; ++i) {
-                S[i] = W[i] * S[i] - AU[i] * us + K[i] * v;
-                acc += S[i] * R[i];
+                for (int e = 0; e < PER_LANE; ++e) {
+                    const int idx = e * 64 + threadIdx.x;
+                    if (idx < 5 * DK) vec[turn][b][idx / DK * VEC + idx % DK / SL * SLP + idx % SL] = next[b][e];
+                }
             }
-            acc += __shfl_xor(acc, 16, WAVE);
-            acc += __shfl_xor(acc, 32, WAVE);
-            if (live && g == 0) o[(size_t)t * heads * dv + h * dv + j] = acc;
+            __syncthreads();                                  // (the buffer of two turns ago was last read before the barrier of the turn between)
+            if (t + TB < t1) fetch(t + TB);
+#pragma unroll
+            for (int b = 0; b < TB; ++b) {
+                if (t + b >= t1) break;
+                const float *W = vec[turn][b] + g * SLP, *AU = W + VEC, *U = W + 2 * VEC, *K = W + 3 * VEC, *R = W + 4 * VEC;
+                // four sums side by side in each pass (added in a fixed order): one chain of SL dependent additions
+                // would be most of a token's time
+                float us4[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int i = 0; i < SL; ++i) us4[i & 3] += U[i] * S[i];
+                const float us = sum_over_groups<SCAN_GROUPS>((us4[0] + us4[1]) + (us4[2] + us4[3]));
+                float acc4[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int i = 0; i < SL; ++i) {
+                    S[i] = W[i] * S[i] - AU[i] * us + K[i] * v[b];
+                    acc4[i & 3] += S[i] * R[i];
+                }
+                const float acc = sum_over_groups<SCAN_GROUPS>((acc4[0] + acc4[1]) + (acc4[2] + acc4[3]));
+                if (live && g == 0) o[(size_t)(t + b) * heads * dv + h * dv + j] = acc;
+            }
         }
         if (live) {
 #pragma unroll
@@ -181,7 +212,7 @@ static int delta_rule_t(const T *proj, int row_stride, int off_r, int off_k, int
     if (threads > 256) threads = 256;
     delta_prep_kernel<T><<<dim3(n, heads), dim3(threads), 0, stream>>>(proj, row_stride, off_r, off_k, off_a, off_l, w2, w0, a_bias, prep, heads, dk, rank);
     LCU_LAUNCH_CHECK();
-#define SCAN(DK) delta_scan_kernel<T, DK><<<dim3(n_req, heads, (dv + (DK ? SCAN_COLS : 64) - 1) / (DK ? SCAN_COLS : 64)), dim3(64), 0, stream>>>(proj, row_stride, off_v, prep, state, o, q_start, ctx_len, state_slot, heads, dk, dv)
+#define SCAN(DK) delta_scan_kernel<T, DK><<<dim3(n_req, heads, (dv + (DK ? 64 / scan_groups<T, DK>() : 64) - 1) / (DK ? 64 / scan_groups<T, DK>() : 64)), dim3(64), 0, stream>>>(proj, row_stride, off_v, prep, state, o, q_start, ctx_len, state_slot, heads, dk, dv)
     switch (dk) {
     case 16: SCAN(16); break;
     case 32: SCAN(32); break;
@@ -202,7 +233,7 @@ static int delta_rule_t(const T *proj, int row_stride, int off_r, int off_k, int
     return LCU_OK;
 }
 
-// proj: [n, row_stride] of `type`; the offsets are columns.  w2: [heads * dk, rank], w0, a_bias: [heads * dk],
+// proj: [n, row_stride] of `type`; the offsets are columns.  w2: [rank, heads * dk] (transposed), w0, a_bias: [heads * dk],
 // weight: [heads * dv], all 32-bit.  prep: scratch [n, heads, 5, dk], o: scratch [n, heads * dv], both 32-bit.
 // state: [slots, heads, dk, dv] 32-bit.  out: [n, heads * dv] of `type`.
 LCU_API int lcu_delta_rule(const void *proj, int type, int row_stride, int off_r, int off_k, int off_v, int off_g,
@@ -211,7 +242,7 @@ LCU_API int lcu_delta_rule(const void *proj, int type, int row_stride, int off_r
                            const int *ctx_len, const int *state_slot, int n, int n_req, int heads, int dk, int dv,
                            int rank, float eps, hipStream_t stream) {
     if (n <= 0 || n_req <= 0) return LCU_OK;
-    if (heads <= 0 || heads > 65535 || dk <= 0 || dv <= 0 || rank <= 0 || rank > MAX_RANK || dv > 16 * 65535) return LCU_BAD_ARGUMENT;
+    if (heads <= 0 || heads > 65535 || dk <= 0 || dv <= 0 || rank <= 0 || rank > MAX_RANK || dv > 8 * 65535) return LCU_BAD_ARGUMENT;
     if (type == LCU_F32)
         return delta_rule_t<float>((const float *)proj, row_stride, off_r, off_k, off_v, off_g, off_a, off_l, w2, w0, a_bias, weight, prep, o, state, (float *)out, q_start, ctx_len, state_slot, n, n_req, heads, dk, dv, rank, eps, stream);
     if (type == LCU_BF16)

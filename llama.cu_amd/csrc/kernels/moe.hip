@@ -193,7 +193,7 @@ __device__ __forceinline__ void moe_store(const f32x4 &acc, int dst, int col0, i
 }
 
 // Few rows an expert (decoding): tiles of up to 16 rows; a block of four waves takes a tile and 64
-// features, a wave 16 of them, and streams its 16 rows of the weight once, four steps of loads in flight.
+// features, a wave 16 of them, and streams its 16 rows of the weight once, eight steps of loads in flight.
 template <class T, int MODE>
 __global__ void __launch_bounds__(256)
 moe_gemm_few_kernel(const T *__restrict__ x, int x_stride, const T *__restrict__ w, size_t w_expert_stride, int N, int K,
@@ -220,14 +220,15 @@ moe_gemm_few_kernel(const T *__restrict__ x, int x_stride, const T *__restrict__
     f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
     const int kfull = K / M::KSTEP * M::KSTEP;
     int k0 = 0;
-    for (; k0 + 4 * M::KSTEP <= kfull; k0 += 4 * M::KSTEP) {
-        frag a[4], b[4];
+    constexpr int AHEAD = 8;                         // steps of loads in flight: a wave's own arithmetic is short
+    for (; k0 + AHEAD * M::KSTEP <= kfull; k0 += AHEAD * M::KSTEP) {
+        frag a[AHEAD], b[AHEAD];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) a[u] = __builtin_nontemporal_load((const frag *)(wrow + k0 + u * M::KSTEP));
+        for (int u = 0; u < AHEAD; ++u) a[u] = __builtin_nontemporal_load((const frag *)(wrow + k0 + u * M::KSTEP));
 #pragma unroll
-        for (int u = 0; u < 4; ++u) b[u] = M::load(xrow + k0 + u * M::KSTEP);
+        for (int u = 0; u < AHEAD; ++u) b[u] = M::load(xrow + k0 + u * M::KSTEP);
 #pragma unroll
-        for (int u = 0; u < 4; ++u) acc = M::mma(a[u], MODE == MOE_UP ? M::scaled(b[u], sc) : b[u], acc);
+        for (int u = 0; u < AHEAD; ++u) acc = M::mma(a[u], MODE == MOE_UP ? M::scaled(b[u], sc) : b[u], acc);
     }
     for (; k0 < K; k0 += M::KSTEP) {                 // the steps that are left, the last one perhaps in part
         const bool in = k0 + g * M::PER_LANE < K;

@@ -47,6 +47,48 @@ layernorm_kernel(float *__restrict__ x, const TD *__restrict__ delta, int planes
     }
 }
 
+// The same for rows of up to NC_THREADS * PT elements: the row stays in registers between its one read and
+// its writes (a step of few rows is a chain of dependent trips to memory, and this kernel has one, not three).
+template <class TD, class TO, int PT>
+__global__ void __launch_bounds__(NC_THREADS)
+layernorm_row_kernel(float *__restrict__ x, const TD *__restrict__ delta, int planes, size_t plane_stride,
+                     const float *__restrict__ w1, const float *__restrict__ b1, TO *__restrict__ out1,
+                     const float *__restrict__ w2, const float *__restrict__ b2, TO *__restrict__ out2, int d, float eps) {
+    __shared__ float scratch[16];
+    float *xr = x + (size_t)blockIdx.x * d;
+    float v[PT], sum = 0.f;
+#pragma unroll
+    for (int i = 0; i < PT; ++i) {
+        const int c = threadIdx.x + NC_THREADS * i;
+        v[i] = 0.f;
+        if (c < d) {
+            v[i] = xr[c];
+            if (delta) {
+                for (int p = 0; p < planes; ++p) v[i] += to_f32(delta[p * plane_stride + (size_t)blockIdx.x * d + c]);
+                xr[c] = v[i];
+            }
+            sum += v[i];
+        }
+    }
+    const float mean = block_sum(sum, scratch) / (float)d;
+    float sq = 0.f;
+#pragma unroll
+    for (int i = 0; i < PT; ++i) {
+        const float dev = v[i] - mean;
+        if (threadIdx.x + NC_THREADS * i < d) sq += dev * dev;
+    }
+    const float rstd = rsqrtf(block_sum(sq, scratch) / (float)d + eps);
+#pragma unroll
+    for (int i = 0; i < PT; ++i) {
+        const int c = threadIdx.x + NC_THREADS * i;
+        if (c < d) {
+            const float z = (v[i] - mean) * rstd;
+            out1[(size_t)blockIdx.x * d + c] = from_f32<TO>(z * w1[c] + b1[c]);
+            if (w2) out2[(size_t)blockIdx.x * d + c] = from_f32<TO>(z * w2[c] + b2[c]);
+        }
+    }
+}
+
 // delta_type: -1 none, LCU_F32 or LCU_BF16.  out_type: LCU_F32 or LCU_BF16.
 LCU_API int lcu_layernorm(float *x, const void *delta, int delta_type, int planes, const float *w1, const float *b1,
                           void *out1, const float *w2, const float *b2, void *out2, int out_type, int n, int d,
@@ -55,13 +97,21 @@ LCU_API int lcu_layernorm(float *x, const void *delta, int delta_type, int plane
     if (d <= 0 || !w1 || !b1 || !out1 || (w2 && (!b2 || !out2)) || (delta && planes <= 0)) return LCU_BAD_ARGUMENT;
     const size_t stride = (size_t)n * d;
     dim3 grid(n), block(NC_THREADS);
-#define GO(TD, TO) layernorm_kernel<TD, TO><<<grid, block, 0, stream>>>(x, (const TD *)delta, planes, stride, w1, b1, (TO *)out1, w2, b2, (TO *)out2, d, eps)
+#define ROW(TD, TO, PT) layernorm_row_kernel<TD, TO, PT><<<grid, block, 0, stream>>>(x, (const TD *)delta, planes, stride, w1, b1, (TO *)out1, w2, b2, (TO *)out2, d, eps)
+#define GO(TD, TO)                                                                                                           \
+    do {                                                                                                                     \
+        if (d <= 4 * NC_THREADS) ROW(TD, TO, 4);                                                                             \
+        else if (d <= 16 * NC_THREADS) ROW(TD, TO, 16);                                                                      \
+        else layernorm_kernel<TD, TO><<<grid, block, 0, stream>>>(x, (const TD *)delta, planes, stride, w1, b1, (TO *)out1,  \
+                                                                  w2, b2, (TO *)out2, d, eps);                               \
+    } while (0)
     const int dt = delta ? delta_type : LCU_F32;
     if (dt == LCU_F32 && out_type == LCU_F32) GO(float, float);
     else if (dt == LCU_F32 && out_type == LCU_BF16) GO(float, bf16_t);
     else if (dt == LCU_BF16 && out_type == LCU_F32) GO(bf16_t, float);
     else if (dt == LCU_BF16 && out_type == LCU_BF16) GO(bf16_t, bf16_t);
     else return LCU_BAD_ARGUMENT;
+#undef ROW
 #undef GO
     LCU_LAUNCH_CHECK();
     return LCU_OK;

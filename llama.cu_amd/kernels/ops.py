@@ -1065,23 +1065,23 @@ def qk_norm_store(qkv: torch.Tensor, positions: torch.Tensor, n_heads: int, n_kv
 # ------------------------------------------------------------------ the generalised delta rule
 
 
-def delta_rule(proj: torch.Tensor, offsets: Dict[str, int], w2: torch.Tensor, w0: torch.Tensor, a_bias: torch.Tensor,
+def delta_rule(proj: torch.Tensor, offsets: Dict[str, int], w2_t: torch.Tensor, w0: torch.Tensor, a_bias: torch.Tensor,
                weight: torch.Tensor, state: torch.Tensor, step, heads: int, key_dim: int, value_dim: int, eps: float,
                out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """The recurrent mixer ``S <- diag(w) S - (a u)(u^T S) + k v^T``, ``o = S^T r`` over the step's rows, request by
     request from each request's state (``state [slots, heads, key_dim, value_dim]`` float32, taken as zero at a
     request's position 0 and left as the step's last token makes it).  ``proj [n, *]`` holds the projections at the
     columns ``offsets``: ``r, k, v, g, a`` (heads * dim each) and ``l`` (the low-rank projection whose ``tanh``,
-    times ``w2 [heads * key_dim, rank]`` plus ``w0``, gives the decay ``w = exp(-exp(-1/2) sigmoid(.))``); ``a =
+    times ``w2`` (given transposed, ``w2_t [rank, heads * key_dim]``) plus ``w0``, gives the decay ``w = exp(-exp(-1/2) sigmoid(.))``); ``a =
     sigmoid(a_lin + a_bias)``, ``u = k / sqrt(sum k^2 + 1e-6)``.  Returns ``o`` of each head divided by its root mean
     square (``eps``), times ``weight``, times ``sigmoid(g)``, in ``proj``'s type ``[n, heads * value_dim]``."""
-    _gpu(proj, w2, w0, a_bias, weight, state, out)
+    _gpu(proj, w2_t, w0, a_bias, weight, state, out)
     _rows(proj, "delta projections")
     n = proj.shape[0]
     hk, hv = heads * key_dim, heads * value_dim
-    if w2.dim() != 2 or w2.shape[0] != hk or w2.dtype != torch.float32 or not w2.is_contiguous():
-        raise KernelError(f"delta_rule: w2 must be contiguous float32 [{hk}, rank], got {w2.dtype} {tuple(w2.shape)}")
-    rank = w2.shape[1]
+    if w2_t.dim() != 2 or w2_t.shape[1] != hk or w2_t.dtype != torch.float32 or not w2_t.is_contiguous():
+        raise KernelError(f"delta_rule: w2_t must be contiguous float32 [rank, {hk}], got {w2_t.dtype} {tuple(w2_t.shape)}")
+    rank = w2_t.shape[0]
     _f32_vec(w0, "delta_rule w0", hk); _f32_vec(a_bias, "delta_rule a_bias", hk); _f32_vec(weight, "delta_rule weight", hv)
     widths = {"r": hk, "k": hk, "v": hv, "g": hv, "a": hk, "l": rank}
     for name, width in widths.items():
@@ -1101,7 +1101,7 @@ def delta_rule(proj: torch.Tensor, offsets: Dict[str, int], w2: torch.Tensor, w0
     o = torch.empty((n, hv), dtype=torch.float32, device=proj.device)
     lib = build.load("delta_rule")
     _check(lib.lcu_delta_rule(_ptr(proj), _type(proj, "delta projections"), proj.stride(0), offsets["r"], offsets["k"], offsets["v"],
-                              offsets["g"], offsets["a"], offsets["l"], _ptr(w2), _ptr(w0), _ptr(a_bias), _ptr(weight), _ptr(prep),
+                              offsets["g"], offsets["a"], offsets["l"], _ptr(w2_t), _ptr(w0), _ptr(a_bias), _ptr(weight), _ptr(prep),
                               _ptr(o), _ptr(state), _ptr(out), _ptr(step.q_start), _ptr(step.ctx_len), _ptr(step.state_slot), n,
                               step.n_req, heads, key_dim, value_dim, rank, ctypes.c_float(eps), _stream()), "delta_rule")
     return out

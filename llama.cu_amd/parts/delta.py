@@ -67,7 +67,7 @@ class GeneralDelta(Part):
         self.offsets = {"r": 0, "k": hd, "v": 2 * hd, "g": 3 * hd, "a": 4 * hd, "l": 5 * hd}
         self.w_o = Weight(tensors[nm["o"]], build)
         # what enters the recurrence is 32-bit: the kernels take these in 32-bit whatever the file holds
-        self.w2 = tensors[nm["w2"]].float().contiguous()
+        self.w2 = tensors[nm["w2"]].float().t().contiguous()        # [rank, heads * dim]: the kernel's lanes read neighbours
         self.w0 = tensors[nm["w0"]].float().contiguous()
         self.a_bias = tensors[nm["a_bias"]].float().contiguous()
         self.norm = tensors[nm["norm"]].float().contiguous()

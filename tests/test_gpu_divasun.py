@@ -133,7 +133,7 @@ def test_delta_rule_against_the_recurrence_in_any_cut(dtype, heads, dim, rank):
         return o, S
 
     want, want_state = plain(proj)
-    args = (off, w2.cuda(), w0.cuda(), ab.cuda(), nw.cuda())
+    args = (off, w2.t().contiguous().cuda(), w0.cuda(), ab.cuda(), nw.cuda())
     rel = 2e-4 if dtype == "float32" else 2e-2
     state = torch.full((3, heads, dim, dim), 5.0, device="cuda")
     whole = ops.delta_rule(proj.cuda(), *args, state, hand_step([T], [T], [1]), heads, dim, dim, eps)
