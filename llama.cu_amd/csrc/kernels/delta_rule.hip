@@ -115,14 +115,14 @@ delta_scan_kernel(const T *__restrict__ proj, int row_stride, int off_v, const f
         auto fetch = [&](int t) {
 #pragma unroll
             for (int b = 0; b < TB; ++b) {
-                const int tt = t + b < t1 ? t + b : t1 - 1;
-                const float *p = prep + ((size_t)tt * heads + h) * 5 * DK;
+                if (t + b >= t1) break;                       // (a step of one token brings in one token)
+                const float *p = prep + ((size_t)(t + b) * heads + h) * 5 * DK;
 #pragma unroll
                 for (int e = 0; e < PER_LANE; ++e) {
                     const int idx = e * 64 + threadIdx.x;
                     next[b][e] = idx < 5 * DK ? p[idx] : 0.f;
                 }
-                v_next[b] = to_f32(vp[(size_t)tt * row_stride]);
+                v_next[b] = to_f32(vp[(size_t)(t + b) * row_stride]);
             }
         };
         if (t0 < t1) fetch(t0);
@@ -131,6 +131,7 @@ delta_scan_kernel(const T *__restrict__ proj, int row_stride, int off_v, const f
             float v[TB];
 #pragma unroll
             for (int b = 0; b < TB; ++b) {
+                if (t + b >= t1) break;
                 v[b] = v_next[b];
 #pragma unroll
                 for (int e = 0; e < PER_LANE; ++e) {

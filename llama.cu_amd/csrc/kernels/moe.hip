@@ -224,7 +224,7 @@ moe_gemm_few_kernel(const T *__restrict__ x, int x_stride, const T *__restrict__
     for (; k0 + AHEAD * M::KSTEP <= kfull; k0 += AHEAD * M::KSTEP) {
         frag a[AHEAD], b[AHEAD];
 #pragma unroll
-        for (int u = 0; u < AHEAD; ++u) a[u] = __builtin_nontemporal_load((const frag *)(wrow + k0 + u * M::KSTEP));
+        for (int u = 0; u < AHEAD; ++u) a[u] = M::load(wrow + k0 + u * M::KSTEP);    // (through the caches: a load takes half of each line, the next one the other half)
 #pragma unroll
         for (int u = 0; u < AHEAD; ++u) b[u] = M::load(xrow + k0 + u * M::KSTEP);
 #pragma unroll

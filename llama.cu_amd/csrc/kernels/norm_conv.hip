@@ -212,3 +212,111 @@ LCU_API int lcu_short_conv(const void *h, int h_type, long long set_stride_h, co
     }
     return LCU_OK;
 }
+
+// ---------------------------------------------------------------- a step of single tokens: all of the above in one kernel
+// Every request feeds one token (row r is request r's): the residual sum, one or two layer norms, their short
+// convolutions from the requests' states, and the states' update, with the row in registers throughout.  A block
+// is the only reader and writer of its request's state, and a thread of its channels'.
+// out: [sets][n, d] of TO; state: [slots, sets, taps - 1, d]; cw: [sets][d, taps] 32-bit.
+template <class TD, class TO, int PT>
+__global__ void __launch_bounds__(NC_THREADS)
+norm_conv_single_kernel(float *__restrict__ x, const TD *__restrict__ delta, int planes, size_t plane_stride,
+                        const float *__restrict__ w1, const float *__restrict__ b1, const float *__restrict__ w2,
+                        const float *__restrict__ b2, const float *__restrict__ cw, float *__restrict__ st,
+                        TO *__restrict__ out, size_t set_stride_out, const int *__restrict__ ctx_len,
+                        const int *__restrict__ state_slot, int d, int taps, int sets, float eps) {
+    __shared__ float scratch[16];
+    const int r = blockIdx.x;
+    const int pos = ctx_len[r] - 1;                  // the token's position
+    float *xr = x + (size_t)r * d;
+    float v[PT], sum = 0.f;
+#pragma unroll
+    for (int i = 0; i < PT; ++i) {
+        const int c = threadIdx.x + NC_THREADS * i;
+        v[i] = 0.f;
+        if (c < d) {
+            v[i] = xr[c];
+            if (delta) {
+                for (int p = 0; p < planes; ++p) v[i] += to_f32(delta[p * plane_stride + (size_t)r * d + c]);
+                xr[c] = v[i];
+            }
+            sum += v[i];
+        }
+    }
+    const float mean = block_sum(sum, scratch) / (float)d;
+    float sq = 0.f;
+#pragma unroll
+    for (int i = 0; i < PT; ++i) {
+        const float dev = v[i] - mean;
+        if (threadIdx.x + NC_THREADS * i < d) sq += dev * dev;
+    }
+    const float rstd = rsqrtf(block_sum(sq, scratch) / (float)d + eps);
+    constexpr int FUSED_TAPS = 8;                    // the most taps this kernel takes
+    for (int s = 0; s < sets; ++s) {
+        const float *w = s ? w2 : w1, *b = s ? b2 : b1;
+        float *state = st + ((size_t)state_slot[r] * sets + s) * (taps - 1) * d;
+        // everything is read before anything is written: the state's new rows are its old ones, and loads that had to
+        // wait for the stores before them would be a chain of trips to memory
+        float old[PT][FUSED_TAPS - 1], k[PT][FUSED_TAPS], wv[PT], bv[PT];
+#pragma unroll
+        for (int i = 0; i < PT; ++i) {
+            const int c = threadIdx.x + NC_THREADS * i;
+            if (c >= d) continue;
+            wv[i] = w[c];
+            bv[i] = b[c];
+#pragma unroll
+            for (int j = 0; j < FUSED_TAPS; ++j)
+                if (j < taps) k[i][j] = cw[((size_t)s * d + c) * taps + j];
+#pragma unroll
+            for (int j = 0; j < FUSED_TAPS - 1; ++j)      // row j of the state lies taps - 1 - j positions before the token
+                if (j < taps - 1) old[i][j] = pos - (taps - 1 - j) >= 0 ? state[(size_t)j * d + c] : 0.f;
+        }
+#pragma unroll
+        for (int i = 0; i < PT; ++i) {
+            const int c = threadIdx.x + NC_THREADS * i;
+            if (c >= d) continue;
+            const float h = (v[i] - mean) * rstd * wv[i] + bv[i];
+            float acc = h;                            // (the order of short_conv_kernel's additions)
+#pragma unroll
+            for (int j = 0; j < FUSED_TAPS - 1; ++j)
+                if (j < taps - 1) {
+                    acc += k[i][j] * old[i][j];
+                    if (j > 0) state[(size_t)(j - 1) * d + c] = old[i][j];     // row j becomes row j - 1
+                }
+#pragma unroll
+            for (int j = 0; j < FUSED_TAPS; ++j)
+                if (j == taps - 1) acc += k[i][j] * h;
+            if (taps > 1) state[(size_t)(taps - 2) * d + c] = h;
+            out[s * set_stride_out + (size_t)r * d + c] = from_f32<TO>(acc);
+        }
+    }
+}
+
+LCU_API int lcu_norm_conv_single(float *x, const void *delta, int delta_type, int planes, const float *w1, const float *b1,
+                                 const float *w2, const float *b2, const float *cw, float *state, void *out, int out_type,
+                                 const int *ctx_len, const int *state_slot, int n, int d, int taps, int sets, float eps,
+                                 hipStream_t stream) {
+    if (n <= 0) return LCU_OK;
+    if (d <= 0 || d > 8 * NC_THREADS || taps < 1 || taps > 8 || sets < 1 || sets > 2 || !w1 || !b1 || (sets == 2 && (!w2 || !b2)) ||
+        !cw || (taps > 1 && !state) || (delta && planes <= 0))
+        return LCU_BAD_ARGUMENT;
+    const size_t stride = (size_t)n * d;
+    dim3 grid(n), block(NC_THREADS);
+#define ROW(TD, TO, PT) norm_conv_single_kernel<TD, TO, PT><<<grid, block, 0, stream>>>(x, (const TD *)delta, planes, stride, w1, b1, w2, b2, cw, state, (TO *)out, stride, ctx_len, state_slot, d, taps, sets, eps)
+#define GO(TD, TO)                                   \
+    do {                                             \
+        if (d <= 4 * NC_THREADS) ROW(TD, TO, 4);     \
+        else ROW(TD, TO, 8);                         \
+    } while (0)
+    const int dt = delta ? delta_type : LCU_F32;
+    if (dt == LCU_F32 && out_type == LCU_F32) GO(float, float);
+    else if (dt == LCU_F32 && out_type == LCU_BF16) GO(float, bf16_t);
+    else if (dt == LCU_BF16 && out_type == LCU_F32) GO(bf16_t, float);
+    else if (dt == LCU_BF16 && out_type == LCU_BF16) GO(bf16_t, bf16_t);
+    else return LCU_BAD_ARGUMENT;
+#undef ROW
+#undef GO
+    LCU_LAUNCH_CHECK();
+    return LCU_OK;
+}
+

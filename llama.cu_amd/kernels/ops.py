@@ -1027,6 +1027,40 @@ def short_conv(h: torch.Tensor, weight: torch.Tensor, state: torch.Tensor, out: 
     return out
 
 
+def norm_conv_single(x: torch.Tensor, delta: Optional[torch.Tensor], weights, biases, eps: float, conv_weight: torch.Tensor,
+                     state: torch.Tensor, out: torch.Tensor, step) -> torch.Tensor:
+    """For a step in which every request feeds one token: ``layernorm`` (with the residual sum), ``short_conv`` and the
+    states' update in one kernel.  ``weights``, ``biases``: one or two float32 vectors each (the norms of the one or two
+    sets); the rest as in ``short_conv``; ``out [sets, n, d]``."""
+    _gpu(x, delta, conv_weight, state, out, *weights, *biases)
+    _rows(x, "norm input"); _contig(x, "norm input"); _contig(out, "conv out"); _contig(conv_weight, "conv weight"); _contig(state, "conv state")
+    n, d = x.shape
+    sets, taps = conv_weight.shape[0], conv_weight.shape[2]
+    if x.dtype != torch.float32 or conv_weight.dtype != torch.float32 or conv_weight.shape[1] != d or out.shape != (sets, n, d) \
+            or len(weights) != sets or len(biases) != sets or sets not in (1, 2) or d > 2048 or taps > 8:
+        raise KernelError("norm_conv_single: operands do not fit (float32 rows of at most 2048, one or two sets, at most 8 taps)")
+    for v in list(weights) + list(biases):
+        _f32_vec(v, "layernorm weight or bias", d)
+    if not step.decode_only or n != step.n_req:
+        raise KernelError("norm_conv_single: only for a step in which every request feeds one token")
+    if taps > 1 and (state.dtype != torch.float32 or state.dim() != 4 or state.shape[1:] != (sets, taps - 1, d)
+                     or max(step.state_slots, default=0) >= state.shape[0]):
+        raise KernelError(f"norm_conv_single: state must be float32 [slots, {sets}, {taps - 1}, {d}] and hold every request's slot")
+    planes = 0
+    if delta is not None:
+        _contig(delta, "norm delta")
+        if delta.shape[-2:] != (n, d) or delta.dim() not in (2, 3):
+            raise KernelError(f"norm delta: shape {tuple(delta.shape)}, expected [{n}, {d}] or planes of it")
+        planes = delta.shape[0] if delta.dim() == 3 else 1
+    lib = build.load("norm_conv")
+    _check(lib.lcu_norm_conv_single(_ptr(x), _ptr(delta), _type(delta, "norm delta") if delta is not None else -1, planes,
+                                    _ptr(weights[0]), _ptr(biases[0]), _ptr(weights[1] if sets == 2 else None),
+                                    _ptr(biases[1] if sets == 2 else None), _ptr(conv_weight), _ptr(state if taps > 1 else None),
+                                    _ptr(out), _type(out, "conv out"), _ptr(step.ctx_len), _ptr(step.state_slot), n, d, taps, sets,
+                                    ctypes.c_float(eps), _stream()), "norm_conv_single")
+    return out
+
+
 # ------------------------------------------------------------------ norm of whole projections, cache write
 
 

@@ -194,6 +194,14 @@ class ParallelBlock(Part):
         conv = self.taps > 0
         # with a convolution behind them the norms write 32-bit rows, which are rounded once, after the convolution
         mid = torch.float32 if conv else self.dtype
+        if conv and self._pair and step.decode_only and d <= 2048 and self.taps <= 8 and (self.taps == 1 or "conv" in cache.more):
+            # every request feeds one token: sum, norms, convolutions and the states' update are one kernel
+            norms = [self.norm1] + ([self.norm2] if self.norm2 is not None else [])
+            state = cache.more["conv"] if self.taps > 1 else torch.empty((1, self.sets, 0, d), dtype=torch.float32, device=x.device)
+            h = ops.norm_conv_single(x, pending, [p.weight for p in norms], [p.bias for p in norms], self.norm1.eps,
+                                     self.conv_weight, state, torch.empty((self.sets, n, d), dtype=self.dtype, device=x.device), step)
+            out = self.mixer.forward(h[0], step, cache, out_dtype=torch.float32)
+            return self.ffn.forward(h[1], add_to=out) if self.ffn is not None else out
         h = torch.empty((self.sets, n, d), dtype=mid, device=x.device)
         if self._pair:
             two = self.norm2 is not None
