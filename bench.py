@@ -380,6 +380,28 @@ def run_designs(args):
     import torch
     import llama_cu_amd  # noqa: F401
     from llama_cu_amd.engine.engine import Engine
+    if args.designs_one:
+        from llama_cu_amd.engine.runner import ModelRunner
+        design, size, what = args.designs_one.split(":")
+        z = DESIGN_SIZES[size]
+        cfg = divasun_config(z, 4096) if design == "divasun" else llama_like(z, 4096)
+        vocab = cfg.vocab if design == "divasun" else cfg.vocab_size
+        runner = ModelRunner.from_config(cfg, 0, dtype=args.dtype, page_size=args.page_size, max_tokens=64 * 1024, max_seqs=66,
+                                         max_batch_tokens=PREFILL_TOKENS, use_graphs=False)
+        rng = random.Random(0)
+        toks = lambda n: [rng.randrange(vocab) for _ in range(n)]
+        if what == "prefill":
+            for k in range(3):
+                runner.step([k], [toks(PREFILL_TOKENS)])
+                runner.end(k)
+        else:
+            ids = list(range(int(what)))
+            for i in ids:
+                runner.step([i], [toks(512)])
+            for _ in range(10):
+                runner.step(ids, [toks(1) for _ in ids])
+        torch.cuda.synchronize()
+        return 0
     sync = torch.cuda.synchronize
     page, prompt, positions = args.page_size, 512, 4096
     steps, warmup = min(args.steps, 32), min(args.warmup, 8)
@@ -464,6 +486,10 @@ def main() -> int:
                          "scheduler (the workload that goes with --shape llama2-7b --batch 64); arrivals: --batch requests "
                          "decode while a prompt of 16 tokens arrives every second step (host time and the GPU's busy "
                          "fraction per kind of step)")
+    ap.add_argument("--designs-one", metavar="DESIGN:SIZE:WHAT", default=None,
+                    help="with --workload designs, for a profiler: only DESIGN (divasun or llama) at SIZE (w2048, w4096), and "
+                         "only WHAT: 'prefill' (three steps of 2,048 tokens) or a number of requests that decode ten steps over "
+                         "prompts of 512 tokens; steps are launched one kernel at a time, not replayed from graphs")
     ap.add_argument("--no-points", action="store_true", help="skip decoding at batch 1 and 64, the prefill and the check")
     ap.add_argument("--no-check", action="store_true",
                     help="skip the comparison of the benchmarked model's logits with the 32-bit path's (same weights, all layers)")
