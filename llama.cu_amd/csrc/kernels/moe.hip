@@ -20,14 +20,15 @@ typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 
 // ---------------------------------------------------------------- route
-// One block of 256 threads per token.  h: [n, d] of T; router: [experts, d] 32-bit.
-// ids, wts: [n, top].  A wave takes the experts e = wave, wave + 4, ...; with d a multiple of 8 a lane
-// keeps its share of the row (eight neighbouring elements of every 512) in registers for all of them.
+// One block per token (256 threads; 1024 where a step has few tokens, so that more of a token's experts are
+// multiplied side by side).  h: [n, d] of T; router: [experts, d] 32-bit.  ids, wts: [n, top].  A wave takes
+// the experts e = wave, wave + waves, ...; with d a multiple of 8 a lane keeps its share of the row (eight
+// neighbouring elements of every 512) in registers for all of them.
 template <class T> struct alignas(8 * sizeof(T)) Row8 { T v[8]; };
 constexpr int ROUTE_CHUNKS = 8;                  // rows of up to 8 * 512 elements stay in registers
 
-template <class T>
-__global__ void __launch_bounds__(256)
+template <class T, int THREADS>
+__global__ void __launch_bounds__(THREADS)
 moe_route_kernel(const T *__restrict__ h, const float *__restrict__ router, int *__restrict__ ids,
                  float *__restrict__ wts, int d, int experts, int top) {
     __shared__ float z[MOE_MAX_EXPERTS];
@@ -44,7 +45,7 @@ moe_route_kernel(const T *__restrict__ h, const float *__restrict__ router, int 
                 for (int e = 0; e < 8; ++e) x[k][e] = to_f32(in.v[e]);
             }
         }
-        for (int e = wave; e < experts; e += 256 / WAVE) {
+        for (int e = wave; e < experts; e += THREADS / WAVE) {
             const float *w = router + (size_t)e * d;
             float acc = 0.f;
 #pragma unroll
@@ -62,7 +63,7 @@ moe_route_kernel(const T *__restrict__ h, const float *__restrict__ router, int 
             if (lane == 0) z[e] = acc;
         }
     } else {
-        for (int e = wave; e < experts; e += 256 / WAVE) {
+        for (int e = wave; e < experts; e += THREADS / WAVE) {
             const float *w = router + (size_t)e * d;
             float acc = 0.f;
             for (int c = lane; c < d; c += WAVE) acc += to_f32(row[c]) * w[c];
@@ -240,8 +241,8 @@ moe_gemm_few_kernel(const T *__restrict__ x, int x_stride, const T *__restrict__
 }
 
 // Many rows an expert (prompts): tiles of up to 64 rows; a block of four waves takes a tile and 128
-// features.  Rows and weights go through LDS in steps of 128 bytes of k, the next step's loads on their
-// way while one is multiplied; a wave multiplies 32 features with all 64 rows (eight sums).
+// features.  Rows and weights go through LDS (two buffers in turn) in steps of 128 bytes of k, the next
+// step's loads on their way while one is multiplied; a wave multiplies 32 features with all 64 rows (eight sums).
 template <class T, int MODE>
 __global__ void __launch_bounds__(256)
 moe_gemm_many_kernel(const T *__restrict__ x, int x_stride, const T *__restrict__ w, size_t w_expert_stride, int N, int K,
@@ -255,8 +256,8 @@ moe_gemm_many_kernel(const T *__restrict__ x, int x_stride, const T *__restrict_
     constexpr int KS = 128 / sizeof(T);             // elements of k a step
     constexpr int CH = KS / PL;                     // 16-byte pieces of a row a step: 8
     constexpr int LD = KS + PL;                     // a row in LDS, with a piece of padding against bank conflicts
-    __shared__ __attribute__((aligned(16))) T xs[64 * LD];
-    __shared__ __attribute__((aligned(16))) T ws[128 * LD];
+    __shared__ __attribute__((aligned(16))) T xs_[2][64 * LD];        // two buffers in turn: one barrier a step
+    __shared__ __attribute__((aligned(16))) T ws_[2][128 * LD];
     const int tile = blockIdx.x;
     if (tile >= n_tiles[0]) return;
     const int n0 = blockIdx.y * 128;
@@ -301,8 +302,10 @@ moe_gemm_many_kernel(const T *__restrict__ x, int x_stride, const T *__restrict_
 #pragma unroll
         for (int m = 0; m < 4; ++m) acc[ft][m] = f32x4{0.f, 0.f, 0.f, 0.f};
     from_memory(0);
-    for (int k0 = 0; k0 < K; k0 += KS) {
-        __syncthreads();                            // the step before has been read
+    int turn = 0;
+    for (int k0 = 0; k0 < K; k0 += KS, turn ^= 1) {
+        T *xs = xs_[turn], *ws = ws_[turn];
+        // (the buffer was last read two steps ago, and every wave has passed the barrier of the step between since)
 #pragma unroll
         for (int i = 0; i < 2; ++i) *(frag *)(xs + (tid / CH + 32 * i) * LD + ch * PL) = xreg[i];
 #pragma unroll
@@ -361,9 +364,12 @@ LCU_API int lcu_moe_route(const void *h, int type, const float *router, int *ids
                           int top, hipStream_t stream) {
     if (n <= 0) return LCU_OK;
     if (d <= 0 || experts <= 0 || experts > MOE_MAX_EXPERTS || top <= 0 || top > experts) return LCU_BAD_ARGUMENT;
-    if (type == LCU_F32) moe_route_kernel<float><<<dim3(n), dim3(256), 0, stream>>>((const float *)h, router, ids, wts, d, experts, top);
-    else if (type == LCU_BF16) moe_route_kernel<bf16_t><<<dim3(n), dim3(256), 0, stream>>>((const bf16_t *)h, router, ids, wts, d, experts, top);
+    const bool few = n <= 256 && experts > 4;
+#define GO(T, TH) moe_route_kernel<T, TH><<<dim3(n), dim3(TH), 0, stream>>>((const T *)h, router, ids, wts, d, experts, top)
+    if (type == LCU_F32) { if (few) GO(float, 1024); else GO(float, 256); }
+    else if (type == LCU_BF16) { if (few) GO(bf16_t, 1024); else GO(bf16_t, 256); }
     else return LCU_BAD_ARGUMENT;
+#undef GO
     LCU_LAUNCH_CHECK();
     return LCU_OK;
 }

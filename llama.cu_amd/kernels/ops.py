@@ -475,7 +475,7 @@ class AttentionPlan:
         return (self.max_tasks, self.per_wg, self.n_single, self.single_splits)
 
 
-def plan_attention(step, n_heads: int, n_kv_heads: int, window: int = 0) -> Optional[AttentionPlan]:
+def plan_attention(step, n_heads: int, n_kv_heads: int, window: int = 0, biased: bool = False) -> Optional[AttentionPlan]:
     """The AttentionPlan of ``step`` for layers with these heads and this window (one per step and kind of layer,
     kept in ``step.scratch``); None for a step of single tokens only, which needs none.  Called before the step's
     arrays go to the device (``Part.prepare``) it lays its lists into the step's own memory (``step.extra``): their
@@ -483,7 +483,8 @@ def plan_attention(step, n_heads: int, n_kv_heads: int, window: int = 0) -> Opti
     Called later (a step made by hand) it brings its lists to the device itself."""
     if step.decode_only:
         return None
-    lib = build.load("attention_mfma")
+    # (the library whose kernels will run is asked: a model with a bias inside its scores needs the other one for nothing)
+    lib = build.load("attention_mfma_bias" if biased else "attention_mfma")
     tpt = lib.lcu_attention_prefill_tokens_per_task(n_heads, n_kv_heads)
     if tpt <= 0:
         return None
@@ -576,7 +577,7 @@ def paged_attention(q: torch.Tensor, out: torch.Tensor, cache: torch.Tensor, ste
                                 page_size, scale, window, splits, req_list=step.decode_order, head_slopes=head_slopes)
     # a mixed batch: the requests that decode one token go to the decode kernel, the portions
     # to the prefill kernel (each would be slow at the other's work)
-    plan = plan_attention(step, n_heads, n_kv_heads, window)
+    plan = plan_attention(step, n_heads, n_kv_heads, window, biased=head_slopes is not None)
     if plan.n_single:
         attention_decode(q, out, cache, bt, step.q_start, step.ctx_len, plan.n_single, n_heads, n_kv_heads, head_dim, page_size,
                          scale, window, plan.single_splits, req_list=plan.singles, head_slopes=head_slopes)

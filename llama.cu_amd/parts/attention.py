@@ -120,7 +120,7 @@ class Attention(Part):
         page_size = self.own_page_size or self.page_size
         if self.dtype == torch.bfloat16 and (self.position.score_slopes() is None or self.scale > 0) \
                 and self.value_dim == self.head_dim and ops.mfma_attention_refusal(self.dtype, self.heads, self.kv_heads, self.head_dim, page_size) is None:
-            ops.plan_attention(step, self.heads, self.kv_heads, self.window)
+            ops.plan_attention(step, self.heads, self.kv_heads, self.window, biased=self.position.score_slopes() is not None)
 
     # forward(..., into=(residual, norm)) may end with the residual sum and that norm's weight
     # in the output projection and return ScaledRows instead of the branch's output

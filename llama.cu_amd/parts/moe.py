@@ -56,6 +56,12 @@ class SigmoidMoE(Part):
         self.router = tensors[self.router_name].float().contiguous()        # the router is 32-bit
         self.w_up = fused_rows([tensors[k] for k in self._ups()]).view(n, ff, d)
         self.w_down = fused_rows([tensors[k] for k in self._downs()]).view(n, d, ff)
+        if ff % 8:
+            # the products load 16 bytes at a time along k: an expert whose size is no multiple of 8 gets rows of zeros
+            # in its up matrix and the columns of zeros that meet them in its down matrix (gelu(0) = 0: nothing changes)
+            pad = 8 - ff % 8
+            self.w_up = torch.cat([self.w_up, self.w_up.new_zeros(n, pad, d)], dim=1).contiguous()
+            self.w_down = torch.cat([self.w_down, self.w_down.new_zeros(n, d, pad)], dim=2).contiguous()
         self.dtype = build.dtype
 
     def forward(self, h, add_to: Optional[torch.Tensor] = None):

@@ -42,11 +42,11 @@ CFG_A = config(131, 72, [
 ], taps=3, eps=1e-4, scale=3.0)
 RANKS_A = {1: 5, 3: 3}
 
-# sizes that the bfloat16 kernels take (multiples of 8); as many key/value heads as heads; one expert a token
+# sizes that the bfloat16 kernels take (multiples of 8, but for one expert size); as many key/value heads as heads; one expert a token
 CFG_B = config(200, 128, [
     {"type": "general_delta", "mixer": {"heads": 2, "dim": 64}, "mlp": moe(6, 1, 64)},
     {"type": "attention", "mixer": attention(4, 4, 32, 32, 0.18, q_temp=(0.25, 16)), "mlp": moe(6, 2, 32)},
-    {"type": "general_delta", "mixer": {"heads": 4, "dim": 16}, "mlp": moe(3, 1, 48)},
+    {"type": "general_delta", "mixer": {"heads": 4, "dim": 16}, "mlp": moe(3, 1, 44)},
     {"type": "attention", "mixer": attention(4, 4, 32, 32, 0.25, kv_from=1), "mlp": None},
 ], taps=4, eps=1e-5, scale=8.0)
 RANKS_B = {0: 8, 2: 4}
