@@ -45,6 +45,7 @@ __global__ void delta_prep_kernel(const T *__restrict__ proj, int row_stride, in
     for (int i = threadIdx.x; i < dk; i += blockDim.x) {
         const int c = h * dk + i;
         float z = w0[c];
+#pragma unroll 8
         for (int j = 0; j < rank; ++j) z += w2t[(size_t)j * heads * dk + c] * th[j];      // (neighbouring lanes, neighbouring addresses)
         const float w = expf(-DECAY_SCALE * sigmoidf_(z));
         const float a = sigmoidf_(to_f32(row[off_a + c]) + a_bias[c]);
