@@ -60,6 +60,18 @@ CFG_C2 = dict(CFG_C1, canon={"taps": 2})
 RANKS_C = {1: 2}
 
 
+# one kind of mixer only: a model without any pages, and one without any recurrent state
+CFG_D = config(64, 48, [
+    {"type": "general_delta", "mixer": {"heads": 2, "dim": 16}, "mlp": moe(3, 1, 16)},
+    {"type": "general_delta", "mixer": {"heads": 1, "dim": 24}, "mlp": None},
+], taps=3, eps=1e-5, scale=2.0)
+RANKS_D = {0: 3, 1: 6}
+CFG_E = config(64, 48, [
+    {"type": "attention", "mixer": attention(3, 3, 8, 8, 0.5, q_temp=(1.0, 1)), "mlp": None},
+    {"type": "attention", "mixer": attention(3, 3, 8, 8, 0.3, kv_from=0), "mlp": moe(2, 1, 8)},
+], taps=5, eps=1e-5, scale=0.5)
+
+
 def random_weights(cfg: dict, ranks: Dict[int, int], seed: int, sharp_keys: float = 1.0) -> Dict[str, torch.Tensor]:
     """Every tensor of the design for ``cfg`` (``ranks``: the decay's low rank per delta layer), bfloat16-exact
     float32 values.  ``sharp_keys``: the keys' norm weights are multiplied by it, which makes the softmax peaked, so
