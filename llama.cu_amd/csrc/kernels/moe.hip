@@ -200,7 +200,7 @@ __global__ void __launch_bounds__(256)
 moe_gemm_few_kernel(const T *__restrict__ x, int x_stride, const T *__restrict__ w, size_t w_expert_stride, int N, int K,
                     const int *__restrict__ sorted_to_flat, const float *__restrict__ wts,
                     const int *__restrict__ tile_expert, const int *__restrict__ tile_begin,
-                    const int *__restrict__ tile_rows, const int *__restrict__ n_tiles, T *__restrict__ out_t,
+                    const int *__restrict__ tile_rows, const int *__restrict__ n_tiles, int /* max_tiles */, T *__restrict__ out_t,
                     float *__restrict__ out_f, int out_stride, int top, int add) {
     typedef Mma<T> M;
     typedef typename M::frag frag;
@@ -241,14 +241,14 @@ moe_gemm_few_kernel(const T *__restrict__ x, int x_stride, const T *__restrict__
 }
 
 // Many rows an expert (prompts): tiles of up to 64 rows; a block of four waves takes a tile and 128
-// features.  Rows and weights go through LDS (two buffers in turn) in steps of 128 bytes of k, the next
-// step's loads on their way while one is multiplied; a wave multiplies 32 features with all 64 rows (eight sums).
+// features.  Rows and weights go through LDS in steps of 128 bytes of k, the next step's loads on their
+// way while one is multiplied; a wave multiplies 32 features with all 64 rows (eight sums).
 template <class T, int MODE>
 __global__ void __launch_bounds__(256)
 moe_gemm_many_kernel(const T *__restrict__ x, int x_stride, const T *__restrict__ w, size_t w_expert_stride, int N, int K,
                      const int *__restrict__ sorted_to_flat, const float *__restrict__ wts,
                      const int *__restrict__ tile_expert, const int *__restrict__ tile_begin,
-                     const int *__restrict__ tile_rows, const int *__restrict__ n_tiles, T *__restrict__ out_t,
+                     const int *__restrict__ tile_rows, const int *__restrict__ n_tiles, int max_tiles, T *__restrict__ out_t,
                      float *__restrict__ out_f, int out_stride, int top, int add) {
     typedef Mma<T> M;
     typedef typename M::frag frag;
@@ -256,11 +256,15 @@ moe_gemm_many_kernel(const T *__restrict__ x, int x_stride, const T *__restrict_
     constexpr int KS = 128 / sizeof(T);             // elements of k a step
     constexpr int CH = KS / PL;                     // 16-byte pieces of a row a step: 8
     constexpr int LD = KS + PL;                     // a row in LDS, with a piece of padding against bank conflicts
-    __shared__ __attribute__((aligned(16))) T xs_[2][64 * LD];        // two buffers in turn: one barrier a step
-    __shared__ __attribute__((aligned(16))) T ws_[2][128 * LD];
-    const int tile = blockIdx.x;
-    if (tile >= n_tiles[0]) return;
-    const int n0 = blockIdx.y * 128;
+    __shared__ __attribute__((aligned(16))) T xs[64 * LD];
+    __shared__ __attribute__((aligned(16))) T ws[128 * LD];
+    // Workgroups go to the chip's eight dies in turn (workgroup i to die i % 8), and each die has an L2 of its own.  The
+    // tiles of one expert want the same block of its matrix: a die takes the feature blocks die, die + 8, ... and walks
+    // the tiles of each in turn, so that a block of a matrix comes from memory to one die only.
+    const int n_fb = (N + 127) / 128, die = blockIdx.x % 8, at = blockIdx.x / 8;
+    const int fb = die + 8 * (at / max_tiles), tile = at % max_tiles;
+    if (fb >= n_fb || tile >= n_tiles[0]) return;
+    const int n0 = fb * 128;
     const int e = tile_expert[tile], row0 = tile_begin[tile], rows = tile_rows[tile];
     const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE, g = lane / 16, l16 = lane % 16;
     const int ch = tid % CH;                        // this thread's piece of k in every row it copies
@@ -302,10 +306,10 @@ moe_gemm_many_kernel(const T *__restrict__ x, int x_stride, const T *__restrict_
 #pragma unroll
         for (int m = 0; m < 4; ++m) acc[ft][m] = f32x4{0.f, 0.f, 0.f, 0.f};
     from_memory(0);
-    int turn = 0;
-    for (int k0 = 0; k0 < K; k0 += KS, turn ^= 1) {
-        T *xs = xs_[turn], *ws = ws_[turn];
-        // (the buffer was last read two steps ago, and every wave has passed the barrier of the step between since)
+    // (one buffer and two barriers a step: with two buffers in turn and one barrier the kernel was a quarter slower, its
+    // workgroups being fewer on a compute unit)
+    for (int k0 = 0; k0 < K; k0 += KS) {
+        __syncthreads();                            // the step before has been read
 #pragma unroll
         for (int i = 0; i < 2; ++i) *(frag *)(xs + (tid / CH + 32 * i) * LD + ch * PL) = xreg[i];
 #pragma unroll
@@ -395,11 +399,15 @@ LCU_API int lcu_moe_experts(const void *h, int type, const int *ids, const float
     float *down_to = add ? out : y;
     const int per_block = tile_rows == 16 ? 64 : 128;         // features a block takes
     dim3 block(256), gu(max_tiles, (ff + per_block - 1) / per_block), gd(max_tiles, (d + per_block - 1) / per_block);
+    if (tile_rows != 16) {                                    // a flat grid: the kernel shares it out over the dies itself
+        gu = dim3(8 * max_tiles * (((ff + 127) / 128 + 7) / 8));
+        gd = dim3(8 * max_tiles * (((d + 127) / 128 + 7) / 8));
+    }
 #define GO(KERNEL, T)                                                                                                              \
     KERNEL<T, MOE_UP><<<gu, block, 0, stream>>>((const T *)h, d, (const T *)w_up, (size_t)ff * d, ff, d, sorted, wts, t_exp, t_beg, \
-                                                t_rows, n_tiles, (T *)act, nullptr, ff, top, 0);                                    \
+                                                t_rows, n_tiles, max_tiles, (T *)act, nullptr, ff, top, 0);                         \
     KERNEL<T, MOE_DOWN><<<gd, block, 0, stream>>>((const T *)act, ff, (const T *)w_down, (size_t)ff * d, d, ff, sorted, wts, t_exp, \
-                                                  t_beg, t_rows, n_tiles, nullptr, down_to, d, top, add)
+                                                  t_beg, t_rows, n_tiles, max_tiles, nullptr, down_to, d, top, add)
     if (type == LCU_BF16) {
         if (tile_rows == 16) { GO(moe_gemm_few_kernel, bf16_t); } else { GO(moe_gemm_many_kernel, bf16_t); }
     } else {
