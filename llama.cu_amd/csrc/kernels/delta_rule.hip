@@ -2,7 +2,7 @@
 // (key channel, value channel) in 32-bit.  For every token, with per key channel a decay w, a
 // removal rate a, the key k, its unit vector u = k / sqrt(sum(k^2) + 1e-6), the query r, and
 // per value channel v:
-//   S <- diag(w) S - (a * u) (u^T S) + k v^T        (both terms read the old S)
+//   S <- diag(w) S - (a * u) (u^T S) + k v^T        (decay and removal act on S as the token found it)
 //   o  = S^T r
 // Everything that enters the recurrence is 32-bit.  Three kernels:
 //   prep  (parallel over tokens and heads): w, a * u, u, k, r as 32-bit vectors;

@@ -1,10 +1,10 @@
 // A feed-forward of many small experts of which each token uses a few.
 //
 //   route:   z = W_router h (32-bit), the `top` experts with the largest z (ties: the lower
-//            index), each with the weight sigmoid(z) (not renormalised);
+//            index), each with the weight sigmoid(z) (a token's weights are not made to add up to one);
 //   group:   the (token, choice) pairs sorted by expert and cut into tiles of up to 16 or 64 rows of
 //            one expert, on the device (nothing comes back to the host);
-//   up:      act = gelu(W_up[e] (weight * h))    the weight multiplies the expert's INPUT
+//   up:      act = gelu(W_up[e] (weight * h))    the weight scales what goes INTO the expert
 //   down:    y = W_down[e] act, added to the token's output row (32-bit).
 // The products run on the matrix cores: bfloat16 operands with v_mfma_f32_16x16x32_bf16, or
 // true 32-bit with v_mfma_f32_16x16x4_f32; sums are 32-bit.  A row's result depends on that

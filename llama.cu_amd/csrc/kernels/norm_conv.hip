@@ -139,7 +139,7 @@ short_conv_kernel(const TI *__restrict__ h, size_t set_stride_h, const TW *__res
         float acc = to_f32(hs[(size_t)t * d + c]);
         for (int j = 0; j < taps; ++j) {
             const int back = taps - 1 - j;                      // the row `back` positions earlier
-            if (pos - back < 0) continue;                       // before the sequence: zero
+            if (pos - back < 0) continue;                       // no such row: the request starts later
             float v;
             if (t - back >= first) v = to_f32(hs[(size_t)(t - back) * d + c]);
             else v = state[(size_t)(taps - 1 - (first - (t - back))) * d + c];

@@ -1167,7 +1167,7 @@ def moe_route(h: torch.Tensor, router: torch.Tensor, top: int):
 def moe_experts(h: torch.Tensor, ids: torch.Tensor, wts: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor,
                 out: torch.Tensor) -> torch.Tensor:
     """``out[t] += sum over t's experts e of  w_down[e] @ gelu(w_up[e] @ (weight * h[t]))`` (the exact gelu; the
-    weight multiplies the expert's input).  ``w_up [experts, ff, d]``, ``w_down [experts, d, ff]`` in ``h``'s type,
+    weight scales what goes INTO the expert, not what comes out).  ``w_up [experts, ff, d]``, ``w_down [experts, d, ff]`` in ``h``'s type,
     ``out`` float32 ``[n, d]``."""
     _gpu(h, ids, wts, w_up, w_down, out)
     _rows(h, "moe input")

@@ -117,7 +117,7 @@ class ParallelBlock(Part):
 
     ``conv_taps > 0``: what each branch reads, ``h``, is first replaced by ``h + conv(h)``, a causal convolution
     over time on each channel with a weight ``[width, taps]`` and no bias (``conv_tensors`` names the two):
-    ``conv(h)[t] = sum_j w[:, j] * h[t - taps + 1 + j]``, zeros before the sequence's start.  The last ``taps - 1``
+    ``conv(h)[t] = sum_j w[:, j] * h[t - taps + 1 + j]``, rows before a request's first token counting as zeros.  The last ``taps - 1``
     inputs of both branches are state of the request (``own_states``), carried from step to step in 32-bit.
 
     The branches' outputs are float32 and are added to one another before the norm that follows adds them to the

@@ -6,7 +6,7 @@ With the mixer's input ``h`` and, per head, key channels ``i`` and value channel
     w = exp(-exp(-1/2) * sigmoid(W_w2 tanh(W_w1 h) + w0))    decay per head and key channel
     a = sigmoid(W_a h + a_b)                                 removal rate per head and key channel
     u = k / sqrt(sum_i k_i^2 + 1e-6)                          the head's unit key
-    S <- diag(w) S - (a * u) (u^T S) + k v^T                  both terms read the old S
+    S <- diag(w) S - (a * u) (u^T S) + k v^T                  decay and removal both act on S as the token found it
     o = S^T r
 
 Each head's ``o`` is divided by its root mean square, the heads side by side are multiplied by a weight per

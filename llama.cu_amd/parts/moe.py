@@ -1,10 +1,10 @@
 """A feed-forward of many small experts of which every token uses a few.
 
     z = W_router h (32-bit),  s = sigmoid(z)
-    the ``top`` experts with the largest scores are chosen (ties: the lower index), weights s, not renormalised
+    the ``top`` experts with the largest scores are chosen (ties: the lower index), with s itself as weight (the weights of a token are not made to add up to one)
     out = sum over the chosen e of  W_down[e] act(W_up[e] (s_e * h))        act: the exact (erf) gelu
 
-The weight multiplies the expert's INPUT.  Routing, grouping by expert and the experts' products all run on
+The weight scales what goes INTO the expert, not what comes out.  Routing, grouping by expert and the experts' products all run on
 the device (``csrc/kernels/moe.hip``): nothing about which expert a token uses comes back to the host, so a
 step's launches depend on its sizes alone.  The experts' matrices are laid out side by side by the loader, so
 that an expert is an index.

@@ -27,7 +27,7 @@ def rms_unit(x, eps):
 
 
 def short_conv(h, w):
-    """``h + conv(h)``: ``conv(h)[t] = sum_j w[:, j] * h[t - taps + 1 + j]``, zeros before the sequence."""
+    """``h + conv(h)``: ``conv(h)[t] = sum_j w[:, j] * h[t - taps + 1 + j]``, rows before the first count as zeros."""
     T, d = h.shape
     taps = w.shape[1]
     padded = torch.cat([torch.zeros(taps - 1, d, dtype=h.dtype), h], 0)
@@ -99,7 +99,7 @@ def attention(h, P, heads: int, kv_heads: int, dim: int, vdim: int, scale: float
 
 
 def moe(h, P, experts: int, top: int, margins: Optional[list] = None):
-    """Every token's ``top`` experts by sigmoid score; the score multiplies the expert's input.  ``margins`` takes
+    """Every token's ``top`` experts by sigmoid score; the score scales what goes into the expert.  ``margins`` takes
     every token's distance between the last chosen logit and the first that was not (how close the call was)."""
     z = h @ P["router"].T
     s = torch.sigmoid(z)
