@@ -492,3 +492,46 @@ def test_trace_replay_of_the_design(tmp_path):
     wa, wb = plain_logits(cfg, w, a), plain_logits(cfg, w, b)
     assert_close(torch.from_numpy(out0), wa[[0, 32]], REL["float32"])
     assert_close(torch.from_numpy(out1), torch.stack([wa[49], wb[29]]), REL["float32"])
+
+
+def test_the_command_line_writes_a_random_model_generates_from_it_and_replays_a_trace(tmp_path):
+    """``random-model`` writes a folder of the design from a configuration that names the decay's rank; ``generate``
+    continues a prompt from it; ``bin/trace_run`` (the program itself, steps on its standard input) gives the plain
+    model's logits for the folder's weights."""
+    import json
+    import os
+    import subprocess
+
+    import numpy as np
+    from llama_cu_amd.weights import open_safetensors
+    from divasun_common import attention, config, moe
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    cfg = config(288, 96, [
+        {"type": "general_delta", "mixer": {"heads": 2, "dim": 32, "decay_rank": 7}, "mlp": moe(4, 2, 48)},
+        {"type": "attention", "mixer": attention(4, 2, 32, 32, 0.2, q_temp=(0.3, 9)), "mlp": moe(4, 1, 48)},
+    ], taps=3, eps=1e-5, scale=4.0)
+    cfg_path, folder, out = str(tmp_path / "c.json"), str(tmp_path / "m"), str(tmp_path / "out")
+    with open(cfg_path, "w") as f:
+        json.dump(cfg, f)
+    tool = os.path.join(root, "bin", "llama.cu_amd")
+    p = subprocess.run([tool, "random-model", cfg_path, folder, "--seed", "3", "--std", "0.1"], capture_output=True, timeout=300)
+    assert p.returncode == 0, p.stderr.decode()[-2000:]
+    p = subprocess.run([tool, "generate", folder, "--max-steps", "6", "-p", "Hi", "--dtype", "float32", "--max-tokens", "256",
+                        "--max-seqs", "2"], capture_output=True, timeout=300)
+    assert p.returncode == 0, p.stderr.decode()[-2000:]
+    assert p.stdout.startswith(b"Hi") and b"n toks = 6" in p.stderr
+    files = open_safetensors(folder)
+    w = {n: f.tensor(n).float() for f in files for n in f.names()}
+    a, b = tokens_of(288, 30, 60), tokens_of(288, 12, 61)
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": a[:19], "want": [18]}], "end": []},
+             {"step": 1, "entries": [{"id": "a", "tokens": a[19:], "want": [0, 10]}, {"id": "b", "tokens": b, "want": [11]}], "end": ["a"]},
+             {"step": 2, "entries": [{"id": "b", "tokens": [5], "want": [0]}], "end": ["b"]}]
+    p = subprocess.run([os.path.join(root, "bin", "trace_run"), "--model", folder, "--dtype", "float32", "--out", out,
+                        "--max-tokens", "128"], input="\n".join(json.dumps(s) for s in steps).encode(), capture_output=True, timeout=300)
+    assert p.returncode == 0, p.stderr.decode()[-2000:]
+    assert [l for l in p.stdout.decode().splitlines() if l.startswith("done")] == ["done 0", "done 1", "done 2"]
+    wa, wb = plain_logits(cfg, w, a), plain_logits(cfg, w, b + [5])
+    got = [torch.from_numpy(np.fromfile(os.path.join(out, f"{k}.f32"), dtype="<f4").reshape(-1, 288)) for k in range(3)]
+    assert_close(got[0], wa[[18]], REL["float32"])
+    assert_close(got[1], torch.stack([wa[19], wa[29], wb[11]]), REL["float32"])
+    assert_close(got[2], wb[[12]], REL["float32"])
