@@ -1067,12 +1067,14 @@ def norm_conv_single(x: torch.Tensor, delta: Optional[torch.Tensor], weights, bi
 
 def qk_norm_store(qkv: torch.Tensor, positions: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: int, value_dim: int,
                   q_weight: Optional[torch.Tensor], k_weight: Optional[torch.Tensor], eps: float, temp_coef: float,
-                  temp_every: int, cache: Optional[torch.Tensor], slots: Optional[torch.Tensor], page_size: int) -> None:
+                  temp_every: int, cache: Optional[torch.Tensor], slots: Optional[torch.Tensor], page_size: int,
+                  q_count: int = 0, k_count: int = 0) -> None:
     """For attention without a rotation: the queries of ``qkv [n, heads * head_dim (+ kv_heads * (head_dim +
     value_dim))]`` are divided by the root mean square over the whole projection and multiplied by ``q_weight``
     (None: no norm) and by ``1 + temp_coef * ln(floor((p + 1) / temp_every) + 1)`` at position ``p`` (0: no such
     factor), in place; the keys likewise (``k_weight``) on their way into ``cache`` at ``slots``, the values as they
-    are.  ``cache=None``: the rows hold queries only."""
+    are.  ``cache=None``: the rows hold queries only.  ``q_count``, ``k_count``: the number of columns that the
+    means run over, if heads were filled up with columns of zeros (0: all columns)."""
     _gpu(qkv, positions, q_weight, k_weight, cache, slots)
     _rows(qkv, "qkv")
     n = qkv.shape[0]
@@ -1093,7 +1095,8 @@ def qk_norm_store(qkv: torch.Tensor, positions: torch.Tensor, n_heads: int, n_kv
     lib = build.load("qk_norm")
     _check(lib.lcu_qk_norm_store(_ptr(qkv), _type(qkv, "qkv"), n, qkv.stride(0), _ptr(positions), _ptr(slots), _ptr(q_weight),
                                  _ptr(k_weight), _ptr(cache), n_heads, n_kv_heads, head_dim, value_dim, page_size,
-                                 ctypes.c_float(eps), ctypes.c_float(temp_coef), int(temp_every or 1), int(store), _stream()),
+                                 ctypes.c_float(eps), ctypes.c_float(temp_coef), int(temp_every or 1), int(store), int(q_count),
+                                 int(k_count), _stream()),
            "qk_norm_store")
 
 

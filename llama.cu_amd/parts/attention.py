@@ -36,9 +36,8 @@ class Attention(Part):
         position ``p`` is multiplied by ``1 + coef * ln(floor((p + 1) / every) + 1)``."""
         if heads % kv_heads:
             raise ValueError(f"attention: {heads} heads are no multiple of {kv_heads} key/value heads")
-        if head_dim % 8 or head_dim > 256:
-            raise ValueError(f"attention: head_dim {head_dim} is not supported by the kernels "
-                             f"(multiples of 8 up to 256)")
+        if head_dim > 256:
+            raise ValueError(f"attention: head_dim {head_dim} is not supported by the kernels (at most 256)")
         self.hidden_size, self.heads, self.kv_heads, self.head_dim = int(hidden_size), int(heads), int(kv_heads), int(head_dim)
         self.scale = float(scale) if scale is not None else float(head_dim) ** -0.5
         self.window = int(window or 0)
@@ -53,6 +52,10 @@ class Attention(Part):
                 raise ValueError(f"attention: the query temperature's step {every} must be at least 1")
             self.q_temp = (float(coef), int(every))
         self.names = dict(self.NAMES, **(names or {}))
+        # the kernels read keys eight dims at a time: a head size that is no multiple of 8 is filled up with dims of
+        # zeros (rows of zeros in the q and k matrices), which change no score; only without a rotation, whose pairs
+        # would not know of them
+        self.padded_dim = (self.head_dim + 7) // 8 * 8
         self.q_norm = self.k_norm = None
         self.own_page_size = int(page_size or 0)  # tokens per page of this layer's cache; 0: the engine's default
         self.shares_kv = bool(shares_kv)          # reads another layer's keys and values: has q and o only
@@ -74,11 +77,22 @@ class Attention(Part):
         return t
 
     def fused_groups(self, dtype, device):
-        return [] if self.shares_kv else [((self.names["q"], self.names["k"], self.names["v"]), 0)]
+        if self.shares_kv or self.padded_dim != self.head_dim:
+            return []
+        return [((self.names["q"], self.names["k"], self.names["v"]), 0)]
 
     def cache_need(self):
-        return PagedKV(self.kv_heads, self.head_dim, self.window, self.own_page_size,
-                       self.value_dim if self.value_dim != self.head_dim else 0)
+        return PagedKV(self.kv_heads, self.padded_dim, self.window, self.own_page_size,
+                       self.value_dim if self.value_dim != self.padded_dim else 0)
+
+    def _pad_heads(self, t: torch.Tensor, heads: int) -> torch.Tensor:
+        """``t [heads * head_dim, ...]`` with every head filled up to ``padded_dim`` rows with zeros."""
+        if self.padded_dim == self.head_dim:
+            return t
+        rest = t.shape[1:]
+        t = t.reshape(heads, self.head_dim, *rest)
+        fill = t.new_zeros((heads, self.padded_dim - self.head_dim) + tuple(rest))
+        return torch.cat([t, fill], dim=1).reshape(heads * self.padded_dim, *rest).contiguous()
 
     def decode_splits(self, batch: int, max_ctx_len: int) -> int:
         """Into how many parts the decode kernel should cut each request's keys when ``batch``
@@ -87,15 +101,20 @@ class Attention(Part):
 
     def load(self, tensors, build: BuildContext) -> None:
         nm = self.names
+        if self.padded_dim != self.head_dim and self.position.rotary_tables() is not None:
+            raise ValueError(f"attention: head_dim {self.head_dim} is no multiple of 8, which the kernels take only without a rotation")
         if self.shares_kv:
-            self.w_qkv = Weight(tensors[nm["q"]], build)
+            self.w_qkv = Weight(self._pad_heads(tensors[nm["q"]], self.heads), build)
+        elif self.padded_dim != self.head_dim:
+            self.w_qkv = Weight(torch.cat([self._pad_heads(tensors[nm["q"]], self.heads),
+                                           self._pad_heads(tensors[nm["k"]], self.kv_heads), tensors[nm["v"]]]).contiguous(), build)
         else:
             # one matrix with the rows of q, then k, then v: in place where the loader laid them out so
             self.w_qkv = Weight(fused_rows([tensors[nm["q"]], tensors[nm["k"]], tensors[nm["v"]]]), build)
         self.w_o = Weight(tensors[nm["o"]], build)
         if self.norm_eps is not None:            # the kernel takes the norms' weights in 32-bit
-            self.q_norm = tensors[nm["q_norm"]].float().contiguous()
-            self.k_norm = None if self.shares_kv else tensors[nm["k_norm"]].float().contiguous()
+            self.q_norm = self._pad_heads(tensors[nm["q_norm"]].float(), self.heads).contiguous()
+            self.k_norm = None if self.shares_kv else self._pad_heads(tensors[nm["k_norm"]].float(), self.kv_heads).contiguous()
         self.position.load({}, build)
         # a position encoding that is its rotation tables alone (apply() does nothing of its own)
         self._rotation_only = type(self.position).apply is Part.apply
@@ -104,11 +123,11 @@ class Attention(Part):
         if self.dtype == torch.bfloat16:
             # a bfloat16 model whose attention the matrix-core kernels do not take still runs, on the generic
             # kernel: correct, and several times slower over long contexts, so the log says so and why
-            why = ops.mfma_attention_refusal(self.dtype, self.heads, self.kv_heads, self.head_dim, self.own_page_size or self.page_size)
+            why = ops.mfma_attention_refusal(self.dtype, self.heads, self.kv_heads, self.padded_dim, self.own_page_size or self.page_size)
             if why is None and self.position.score_slopes() is not None and not self.scale > 0:
                 why = "with a bias inside the scores the matrix-core kernels need a positive scale"
-            if why is None and self.value_dim != self.head_dim:
-                why = f"the values' head size {self.value_dim} is not the keys' {self.head_dim}"
+            if why is None and self.value_dim != self.padded_dim:
+                why = f"the values' head size {self.value_dim} is not the keys' {self.padded_dim}"
             if why is not None:
                 ops.say_once(f"attention with {self.heads} heads of {self.head_dim} in {self.kv_heads} groups runs on the generic "
                              f"kernel, not on the matrix cores: {why}")
@@ -119,7 +138,7 @@ class Attention(Part):
         the step's sizes alone."""
         page_size = self.own_page_size or self.page_size
         if self.dtype == torch.bfloat16 and (self.position.score_slopes() is None or self.scale > 0) \
-                and self.value_dim == self.head_dim and ops.mfma_attention_refusal(self.dtype, self.heads, self.kv_heads, self.head_dim, page_size) is None:
+                and self.value_dim == self.padded_dim and ops.mfma_attention_refusal(self.dtype, self.heads, self.kv_heads, self.padded_dim, page_size) is None:
             ops.plan_attention(step, self.heads, self.kv_heads, self.window, biased=self.position.score_slopes() is not None)
 
     # forward(..., into=(residual, norm)) may end with the residual sum and that norm's weight
@@ -137,7 +156,7 @@ class Attention(Part):
     def forward(self, h, step, cache, into=None, planes_ok=False, out_dtype=None):
         """``out_dtype``: the type of the branch's output if it is not the compute type (a block that adds
         several branches before the residual sum asks for float32)."""
-        nh, nkv, dh, dv = self.heads, self.kv_heads, self.head_dim, self.value_dim
+        nh, nkv, dh, dv = self.heads, self.kv_heads, self.padded_dim, self.value_dim       # (dh: as the kernels see a head)
         plain = self.norm_eps is None and self.q_temp is None       # nothing but a rotation between the product and the cache
         if not plain and self.position.rotary_tables() is not None:
             raise ops.KernelError("attention: a norm over the whole projection or a query temperature together with a rotation is not supported")
@@ -172,7 +191,8 @@ class Attention(Part):
                 coef, every = self.q_temp or (0.0, 1)
                 ops.qk_norm_store(qkv, step.positions, nh, nkv, dh, dv, self.q_norm, self.k_norm, self.norm_eps or 0.0,
                                   coef, every, cache.pages if store else None,
-                                  step.slots(cache.group) if store else None, page_size)
+                                  step.slots(cache.group) if store else None, page_size,
+                                  q_count=nh * self.head_dim, k_count=nkv * self.head_dim)
         out = torch.empty((n_rows, nh * dv), dtype=self.dtype, device=qkv.device)
         ops.paged_attention(qkv, out, cache.pages, step, cache.group, nh, nkv, dh, page_size, self.scale,
                             self.window, head_slopes=self.position.score_slopes(), value_dim=dv)

@@ -72,6 +72,15 @@ CFG_E = config(64, 48, [
 ], taps=5, eps=1e-5, scale=0.5)
 
 
+# head sizes of the attention that are no multiples of 8 (the engine fills its heads up with dims of zeros): 20 with
+# values of 12; 60, which filled up is a size of the matrix-core kernels, with values of 64
+CFG_F = config(80, 64, [
+    {"type": "attention", "mixer": attention(3, 1, 20, 12, 0.3, q_temp=(0.4, 5)), "mlp": moe(3, 1, 16)},
+    {"type": "attention", "mixer": attention(2, 2, 60, 64, 0.15), "mlp": None},
+    {"type": "attention", "mixer": attention(3, 1, 20, 12, 0.4, kv_from=0), "mlp": moe(2, 2, 24)},
+], taps=2, eps=1e-5, scale=1.5)
+
+
 def random_weights(cfg: dict, ranks: Dict[int, int], seed: int, sharp_keys: float = 1.0) -> Dict[str, torch.Tensor]:
     """Every tensor of the design for ``cfg`` (``ranks``: the decay's low rank per delta layer), bfloat16-exact
     float32 values.  ``sharp_keys``: the keys' norm weights are multiplied by it, which makes the softmax peaked, so

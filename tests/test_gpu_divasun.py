@@ -10,7 +10,7 @@ import pytest
 import torch
 
 import plain_divasun as P
-from divasun_common import (CFG_A, CFG_B, CFG_C1, CFG_C2, CFG_D, CFG_E, RANKS_A, RANKS_B, RANKS_C, RANKS_D, assert_close, make_folder,
+from divasun_common import (CFG_A, CFG_B, CFG_C1, CFG_C2, CFG_D, CFG_E, CFG_F, RANKS_A, RANKS_B, RANKS_C, RANKS_D, assert_close, make_folder,
                             plain_logits, random_weights, safe_tokens, tokens_of)
 
 pytestmark = pytest.mark.gpu
@@ -286,7 +286,7 @@ def model(name, sharp=1.0):
     key = (name, sharp)
     if key not in _made:
         cfg, ranks, seed = {"A": (CFG_A, RANKS_A, 1), "B": (CFG_B, RANKS_B, 2), "C1": (CFG_C1, RANKS_C, 3), "C2": (CFG_C2, RANKS_C, 4),
-                            "D": (CFG_D, RANKS_D, 5), "E": (CFG_E, {}, 6)}[name]
+                            "D": (CFG_D, RANKS_D, 5), "E": (CFG_E, {}, 6), "F": (CFG_F, {}, 7)}[name]
         w = random_weights(cfg, ranks, seed, sharp_keys=sharp)
         _made[key] = (cfg, w, make_folder(cfg, w))
     return _made[key]
@@ -311,14 +311,15 @@ def test_a_whole_prompt_against_the_plain_model(name, dtype):
     r.cache.check()
 
 
-@pytest.mark.parametrize("name", ["D", "E"])
-def test_models_of_one_kind_of_mixer_only(name):
+@pytest.mark.parametrize("name,dtype", [("D", "float32"), ("E", "float32"), ("F", "float32"), ("F", "bfloat16")])
+def test_models_of_one_kind_of_mixer_only_and_head_sizes_that_are_filled_up(name, dtype):
     """Recurrent layers alone (no pages at all) and attention alone (no mixer state): a prompt in portions, then
     tokens one by one, a second request beside the first, a slot used again."""
     cfg, w, folder = model(name)
-    a, b = tokens_of(cfg["vocab"], 40, 50), tokens_of(cfg["vocab"], 21, 51)
+    make = (lambda n, seed: safe_tokens(cfg, w, n, seed)) if dtype == "bfloat16" else (lambda n, seed: tokens_of(cfg["vocab"], n, seed))
+    a, b = make(40, 50), make(21, 51)
     wa, wb = plain_logits(cfg, w, a), plain_logits(cfg, w, b)
-    r = runner_for(folder, "float32", max_seqs=2, max_tokens=128)
+    r = runner_for(folder, dtype, max_seqs=2, max_tokens=128)
     got_a = [r.step([0], [a[:17]], [list(range(17))]).clone()]
     out = r.step([0, 1], [a[17:30], b[:20]], [list(range(13)), list(range(20))]).clone()
     got_a.append(out[:13])
@@ -327,10 +328,10 @@ def test_models_of_one_kind_of_mixer_only(name):
     got_b.append(out[:1]); got_a.append(out[1:])
     r.end(1)
     got_a += [r.step([0], [[t]], [[0]]).clone() for t in a[31:]]
-    assert_close(torch.cat(got_a), wa, REL["float32"], "first request")
-    assert_close(torch.cat(got_b), wb, REL["float32"], "second request")
+    assert_close(torch.cat(got_a), wa, REL[dtype], "first request")
+    assert_close(torch.cat(got_b), wb, REL[dtype], "second request")
     again = r.step([2], [b], [list(range(21))])          # in the slot (and pages) that the second request held
-    assert_close(again, wb, REL["float32"], "the slot used again")
+    assert_close(again, wb, REL[dtype], "the slot used again")
     r.cache.check()
 
 
