@@ -3,8 +3,9 @@
 // size that is a multiple of 8, a window or none), for 32-bit and bfloat16 storage.
 //
 // One wave per (token, head).  A token's request, its absolute position p and the
-// keys it sees, [lo, p] with lo = max(0, p - window + 1) (0 without a window), come
-// from the batch arrays.  Keys are walked in chunks of 64 that start at multiples of
+// keys it sees, [lo, p] with lo = max(0, p - window + 1) (0 without a window; with
+// chunk > 0 instead lo = p - p % chunk: the keys of the query's own chunk, chunks counted
+// from the request's position 0), come from the batch arrays.  Keys are walked in chunks of 64 that start at multiples of
 // 64, a lane per key; scores, the running maximum and sum (online softmax) and the
 // output are 32-bit.  What a (token, head) computes, and the order it adds in,
 // depends on p and the cache's contents only: not on how the step's tokens were cut,
@@ -24,11 +25,11 @@ paged_attention_generic_kernel(const T *__restrict__ q, int q_stride, T *__restr
                                const T *__restrict__ cache, const int *__restrict__ block_table, int max_pages,
                                const int *__restrict__ q_start, const int *__restrict__ ctx_len,
                                const int *__restrict__ req_of_token, int nh, int nkvh, int dh, int dv, int page,
-                               float scale, int window, const float *__restrict__ head_slopes) {
+                               float scale, int window, int chunk, const float *__restrict__ head_slopes) {
     const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
     const int r = req_of_token[t];
     const int p = ctx_len[r] - (q_start[r + 1] - t);
-    const int lo = window > 0 ? (p - window + 1 > 0 ? p - window + 1 : 0) : 0;
+    const int lo = chunk > 0 ? p - p % chunk : window > 0 ? (p - window + 1 > 0 ? p - window + 1 : 0) : 0;
     const int kvh = h / (nh / nkvh);
     const int dh8 = dh / 8;
     const float slope = head_slopes ? head_slopes[h] : 0.f;
@@ -98,16 +99,16 @@ LCU_API int lcu_paged_attention_generic(const void *q, int q_stride, void *out, 
                                         const void *cache, const int *block_table, int max_pages,
                                         const int *q_start, const int *ctx_len, const int *req_of_token, int n,
                                         int nh, int nkvh, int dh, int dv, int page, float scale, int window,
-                                        const float *head_slopes, hipStream_t stream) {
+                                        int chunk, const float *head_slopes, hipStream_t stream) {
     if (n <= 0) return LCU_OK;
     if (nh <= 0 || nkvh <= 0 || nh % nkvh || dh <= 0 || dh % 8 || dh > MAX_HEAD_DIM || dv <= 0 || dv > MAX_HEAD_DIM || page <= 0 || page % 8 ||
-        max_pages <= 0 || window < 0 || nh > 65535)
+        max_pages <= 0 || window < 0 || chunk < 0 || (window > 0 && chunk > 0) || nh > 65535)
         return LCU_BAD_ARGUMENT;
     dim3 grid(n, nh), block(WAVE);
     if (type == LCU_F32)
-        paged_attention_generic_kernel<float><<<grid, block, 0, stream>>>((const float *)q, q_stride, (float *)out, out_stride, (const float *)cache, block_table, max_pages, q_start, ctx_len, req_of_token, nh, nkvh, dh, dv, page, scale, window, head_slopes);
+        paged_attention_generic_kernel<float><<<grid, block, 0, stream>>>((const float *)q, q_stride, (float *)out, out_stride, (const float *)cache, block_table, max_pages, q_start, ctx_len, req_of_token, nh, nkvh, dh, dv, page, scale, window, chunk, head_slopes);
     else if (type == LCU_BF16)
-        paged_attention_generic_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t *)q, q_stride, (bf16_t *)out, out_stride, (const bf16_t *)cache, block_table, max_pages, q_start, ctx_len, req_of_token, nh, nkvh, dh, dv, page, scale, window, head_slopes);
+        paged_attention_generic_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t *)q, q_stride, (bf16_t *)out, out_stride, (const bf16_t *)cache, block_table, max_pages, q_start, ctx_len, req_of_token, nh, nkvh, dh, dv, page, scale, window, chunk, head_slopes);
     else
         return LCU_BAD_ARGUMENT;
     LCU_LAUNCH_CHECK();

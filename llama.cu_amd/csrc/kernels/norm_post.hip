@@ -1,0 +1,94 @@
+// A norm BEHIND a sublayer, the residual sum, and the norm in front of the next sublayer, in one pass:
+//
+//   x <- x + a * rsqrt(mean(a^2) + eps_post) * w_post          (a: the sublayer's output; x: the 32-bit residual stream)
+//   h  = x * rsqrt(mean(x^2) + eps_pre) * w_pre                (only if w_pre is given)
+//
+// One block per row; sums, factors and the stream are 32-bit, one rounding where h is stored.  The weights are the
+// factors themselves (a model that stores them around zero adds the one when it loads them).  The order of the sums
+// depends on the width and the block size only.
+#include "common.h"
+
+constexpr int NP_THREADS = 256;
+constexpr int NP_KEEP = 8;          // elements of a row that a thread keeps in registers: rows up to 2048 are read once
+
+template <class TA, class TO>
+__global__ void __launch_bounds__(NP_THREADS)
+norm_post_kernel(float *__restrict__ x, const TA *__restrict__ a, const float *__restrict__ w_post, float eps_post,
+                 const float *__restrict__ w_pre, float eps_pre, TO *__restrict__ out, int d) {
+    __shared__ float scratch[16];
+    float *xr = x + (size_t)blockIdx.x * d;
+    const TA *ar = a + (size_t)blockIdx.x * d;
+    float keep[NP_KEEP];
+    float acc = 0.f;
+#pragma unroll
+    for (int e = 0; e < NP_KEEP; ++e) {
+        const int c = threadIdx.x + e * NP_THREADS;
+        keep[e] = c < d ? to_f32(ar[c]) : 0.f;
+        acc += keep[e] * keep[e];
+    }
+    for (int c = threadIdx.x + NP_KEEP * NP_THREADS; c < d; c += NP_THREADS) {
+        const float v = to_f32(ar[c]);
+        acc += v * v;
+    }
+    const float f_post = rsqrtf(block_sum(acc, scratch) / (float)d + eps_post);
+    acc = 0.f;
+#pragma unroll
+    for (int e = 0; e < NP_KEEP; ++e) {
+        const int c = threadIdx.x + e * NP_THREADS;
+        if (c < d) {
+            keep[e] = xr[c] + keep[e] * f_post * w_post[c];
+            xr[c] = keep[e];
+            acc += keep[e] * keep[e];
+        }
+    }
+    for (int c = threadIdx.x + NP_KEEP * NP_THREADS; c < d; c += NP_THREADS) {
+        const float v = xr[c] + to_f32(ar[c]) * f_post * w_post[c];
+        xr[c] = v;
+        acc += v * v;
+    }
+    if (!w_pre) return;
+    const float f_pre = rsqrtf(block_sum(acc, scratch) / (float)d + eps_pre);
+    TO *o = out + (size_t)blockIdx.x * d;
+#pragma unroll
+    for (int e = 0; e < NP_KEEP; ++e) {
+        const int c = threadIdx.x + e * NP_THREADS;
+        if (c < d) o[c] = from_f32<TO>(keep[e] * f_pre * w_pre[c]);
+    }
+    for (int c = threadIdx.x + NP_KEEP * NP_THREADS; c < d; c += NP_THREADS)      // (a thread reads what it wrote itself)
+        o[c] = from_f32<TO>(xr[c] * f_pre * w_pre[c]);
+}
+
+// x: [n, d] float32, updated in place.  a: [n, d] of a_type.  w_post, w_pre: float32 [d]; w_pre (and out) may be null.
+LCU_API int lcu_norm_post(float *x, const void *a, int a_type, const float *w_post, float eps_post, const float *w_pre,
+                          float eps_pre, void *out, int out_type, int n, int d, hipStream_t stream) {
+    if (n <= 0) return LCU_OK;
+    if (d <= 0 || !x || !a || !w_post || (w_pre && !out)) return LCU_BAD_ARGUMENT;
+    dim3 grid(n), block(NP_THREADS);
+#define GO(TA, TO) norm_post_kernel<TA, TO><<<grid, block, 0, stream>>>(x, (const TA *)a, w_post, eps_post, w_pre, eps_pre, (TO *)out, d)
+    if (a_type == LCU_F32 && out_type == LCU_F32) GO(float, float);
+    else if (a_type == LCU_F32 && out_type == LCU_BF16) GO(float, bf16_t);
+    else if (a_type == LCU_BF16 && out_type == LCU_BF16) GO(bf16_t, bf16_t);
+    else if (a_type == LCU_BF16 && out_type == LCU_F32) GO(bf16_t, float);
+    else return LCU_BAD_ARGUMENT;
+#undef GO
+    LCU_LAUNCH_CHECK();
+    return LCU_OK;
+}
+
+// acc = (first ? 0 : acc) + scale * x over `count` floats: the 32-bit sum of several branches' outputs.
+template <class TX>
+__global__ void scaled_sum_kernel(float *__restrict__ acc, const TX *__restrict__ x, float scale, long long count, int first) {
+    const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < count) acc[i] = (first ? 0.f : acc[i]) + scale * to_f32(x[i]);
+}
+
+LCU_API int lcu_scaled_sum(float *acc, const void *x, int x_type, float scale, long long count, int first, hipStream_t stream) {
+    if (count <= 0) return LCU_OK;
+    if (!acc || !x) return LCU_BAD_ARGUMENT;
+    dim3 grid((unsigned)((count + 255) / 256)), block(256);
+    if (x_type == LCU_F32) scaled_sum_kernel<float><<<grid, block, 0, stream>>>(acc, (const float *)x, scale, count, first);
+    else if (x_type == LCU_BF16) scaled_sum_kernel<bf16_t><<<grid, block, 0, stream>>>(acc, (const bf16_t *)x, scale, count, first);
+    else return LCU_BAD_ARGUMENT;
+    LCU_LAUNCH_CHECK();
+    return LCU_OK;
+}

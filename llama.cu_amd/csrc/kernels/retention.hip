@@ -1,0 +1,152 @@
+// Retention: linear attention with a fixed decay per head, no softmax and no denominator.  Per head, with key
+// channels i and value channels j, a state S [d, dv] in 32-bit:
+//
+//   q, k <- the first rot_dim dims turned by the angle of the token's position (tables; pairing as in the
+//           attention's rotation), k then times k_scale
+//   S <- decay[h] * S + k v^T          o = S^T q
+//
+// The scan: a request's tokens are one chain, but column j of S depends on column j alone, so a workgroup takes a
+// tile of 32 columns of one head of one request and keeps them in registers from the request's first token of the
+// step to its last: eight lanes a column, each with every eighth key channel; the sum over key channels crosses the
+// eight lanes at the end of a token.  q, k (rotated, 32-bit) and v go through LDS, RT_TOK tokens at a time.  The state
+// is taken as zero where the request's first token of the step stands at position 0, and is left as the step's
+// last token makes it.  The order of every sum depends on d alone: however a prompt is cut into steps, the same
+// bits come out.
+//
+// The output: each head's o divided by its root mean square (eps, no weight), times silu(gate) (second kernel).
+#include "common.h"
+
+constexpr int RT_THREADS = 256;
+constexpr int RT_LANES = 8;                       // lanes that share a column
+constexpr int RT_COLS = RT_THREADS / RT_LANES;    // columns a workgroup
+constexpr int RT_TOK = 16;                        // tokens staged at a time
+
+template <class TI, int DPL>                      // DPL: key channels per lane (d <= 8 * DPL)
+__global__ void __launch_bounds__(RT_THREADS)
+retention_scan_kernel(const TI *__restrict__ rows, int row_stride, int q_off, int k_off, int v_off,
+                      const int *__restrict__ positions, const float *__restrict__ cos_t, const float *__restrict__ sin_t,
+                      int max_pos, int rot_dim, int pairing, float k_scale, const float *__restrict__ decay,
+                      float *__restrict__ state, float *__restrict__ o_out, const int *__restrict__ q_start,
+                      const int *__restrict__ ctx_len, const int *__restrict__ state_slot, int nh, int d, int dv) {
+    constexpr int D = 8 * DPL;
+    __shared__ float qs[RT_TOK][D], ks[RT_TOK][D], vs[RT_TOK][RT_COLS];
+    const int r = blockIdx.z, h = blockIdx.y, col0 = blockIdx.x * RT_COLS;
+    const int t0 = q_start[r], t1 = q_start[r + 1];
+    if (t1 <= t0) return;
+    const int first_pos = ctx_len[r] - (t1 - t0);
+    const int sub = threadIdx.x % RT_LANES, col = col0 + threadIdx.x / RT_LANES;
+    const bool live = col < dv;
+    float *S = state + ((size_t)state_slot[r] * nh + h) * (size_t)d * dv;
+    const float g = decay[h];
+    float s[DPL];
+#pragma unroll
+    for (int e = 0; e < DPL; ++e) {
+        const int i = sub + RT_LANES * e;
+        s[e] = (live && i < d && first_pos > 0) ? S[(size_t)i * dv + col] : 0.f;
+    }
+    const int half = rot_dim / 2;
+    for (int base = t0; base < t1; base += RT_TOK) {
+        const int nt = min(RT_TOK, t1 - base);
+        __syncthreads();
+        // stage: pairs of q and k (rotated), the rest of the dims, the tile of v
+        for (int w = threadIdx.x; w < nt * D; w += RT_THREADS) {
+            const int tt = w / D, i = w % D, t = base + tt;
+            const TI *row = rows + (size_t)t * row_stride;
+            float qv = 0.f, kv = 0.f;
+            if (i < d) {
+                qv = to_f32(row[q_off + h * d + i]);
+                kv = to_f32(row[k_off + h * d + i]);
+                if (cos_t && i < rot_dim) {
+                    const int pos = positions[t];
+                    int pi, partner;
+                    bool first;                                   // whether i is the pair's first dim
+                    if (pairing == 0) { first = i < half; pi = first ? i : i - half; partner = first ? i + half : i - half; }
+                    else { first = (i & 1) == 0; pi = i >> 1; partner = i ^ 1; }
+                    const float qp = to_f32(row[q_off + h * d + partner]), kp = to_f32(row[k_off + h * d + partner]);
+                    float c = __uint_as_float(0x7fc00000u), sn = c;
+                    if (pos >= 0 && pos < max_pos) { c = cos_t[(size_t)pos * half + pi]; sn = sin_t[(size_t)pos * half + pi]; }
+                    float ra, rb;
+                    if (first) { rotate_pair(qv, qp, c, sn, ra, rb); qv = ra; rotate_pair(kv, kp, c, sn, ra, rb); kv = ra; }
+                    else { rotate_pair(qp, qv, c, sn, ra, rb); qv = rb; rotate_pair(kp, kv, c, sn, ra, rb); kv = rb; }
+                }
+                kv *= k_scale;
+            }
+            qs[tt][i] = qv;
+            ks[tt][i] = kv;
+        }
+        for (int w = threadIdx.x; w < nt * RT_COLS; w += RT_THREADS) {
+            const int tt = w / RT_COLS, c = col0 + w % RT_COLS;
+            vs[tt][w % RT_COLS] = c < dv ? to_f32(rows[(size_t)(base + tt) * row_stride + v_off + h * dv + c]) : 0.f;
+        }
+        __syncthreads();
+        for (int tt = 0; tt < nt; ++tt) {
+            const float v = vs[tt][threadIdx.x / RT_LANES];
+            float acc = 0.f;
+#pragma unroll
+            for (int e = 0; e < DPL; ++e) {
+                const int i = sub + RT_LANES * e;
+                s[e] = g * s[e] + ks[tt][i] * v;
+                acc += s[e] * qs[tt][i];
+            }
+            acc += __shfl_xor(acc, 1, WAVE);
+            acc += __shfl_xor(acc, 2, WAVE);
+            acc += __shfl_xor(acc, 4, WAVE);
+            if (sub == 0 && live) o_out[(size_t)(base + tt) * nh * dv + (size_t)h * dv + col] = acc;
+        }
+    }
+    if (live) {
+#pragma unroll
+        for (int e = 0; e < DPL; ++e) {
+            const int i = sub + RT_LANES * e;
+            if (i < d) S[(size_t)i * dv + col] = s[e];
+        }
+    }
+}
+
+// out[t, h, :] = o[t, h, :] * rsqrt(mean_j o[t, h, j]^2 + eps) * silu(gate[t, h, :]); one wave per (token, head).
+template <class TG, class T>
+__global__ void __launch_bounds__(WAVE)
+retention_out_kernel(const float *__restrict__ o, const TG *__restrict__ gate, int gate_stride, int g_off, T *__restrict__ out,
+                     int nh, int dv, float eps) {
+    const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+    const float *orow = o + (size_t)t * nh * dv + (size_t)h * dv;
+    float sq = 0.f;
+    for (int c = lane; c < dv; c += WAVE) sq += orow[c] * orow[c];
+    const float f = rsqrtf(wave_sum(sq) / (float)dv + eps);
+    for (int c = lane; c < dv; c += WAVE) {
+        const float z = to_f32(gate[(size_t)t * gate_stride + g_off + h * dv + c]);
+        out[(size_t)t * nh * dv + (size_t)h * dv + c] = from_f32<T>(orow[c] * f * (z / (1.0f + expf(-z))));
+    }
+}
+
+// rows: [n, row_stride] of in_type with q (nh * d) at q_off, k at k_off, v (nh * dv) at v_off and the gate (nh * dv)
+// at g_off.  decay: float32 [nh].  state: float32 [slots, nh, d, dv].  o: float32 scratch [n, nh * dv].
+// out: [n, nh * dv] of out_type.  cos_t / sin_t may be null (no rotation).
+LCU_API int lcu_retention(const void *rows, int in_type, int row_stride, int q_off, int k_off, int v_off, int g_off,
+                          const int *positions, const float *cos_t, const float *sin_t, int max_pos, int rot_dim, int pairing,
+                          float k_scale, const float *decay, float *state, float *o, void *out, int out_type,
+                          const int *q_start, const int *ctx_len, const int *state_slot, int n, int n_req, int nh, int d,
+                          int dv, float eps, hipStream_t stream) {
+    if (n <= 0 || n_req <= 0) return LCU_OK;
+    if (nh <= 0 || d <= 0 || d > 256 || dv <= 0 || rot_dim < 0 || rot_dim % 2 || rot_dim > d || (pairing != 0 && pairing != 1) ||
+        !rows || !decay || !state || !o || !out || (cos_t && (!sin_t || !positions)) || nh > 65535 || n_req > 65535)
+        return LCU_BAD_ARGUMENT;
+    dim3 grid((dv + RT_COLS - 1) / RT_COLS, nh, n_req), block(RT_THREADS);
+#define SCAN(TI, DPL) retention_scan_kernel<TI, DPL><<<grid, block, 0, stream>>>((const TI *)rows, row_stride, q_off, k_off, v_off, positions, cos_t, sin_t, max_pos, rot_dim, pairing, k_scale, decay, state, o, q_start, ctx_len, state_slot, nh, d, dv)
+#define BY_DIM(TI) do { if (d <= 32) SCAN(TI, 4); else if (d <= 64) SCAN(TI, 8); else if (d <= 128) SCAN(TI, 16); else SCAN(TI, 32); } while (0)
+    if (in_type == LCU_F32) BY_DIM(float);
+    else if (in_type == LCU_BF16) BY_DIM(bf16_t);
+    else return LCU_BAD_ARGUMENT;
+#undef BY_DIM
+#undef SCAN
+    LCU_LAUNCH_CHECK();
+    dim3 ogrid(n, nh), oblock(WAVE);
+#define OUT(TG, T) retention_out_kernel<TG, T><<<ogrid, oblock, 0, stream>>>(o, (const TG *)rows, row_stride, g_off, (T *)out, nh, dv, eps)
+    if (in_type == LCU_F32 && out_type == LCU_F32) OUT(float, float);
+    else if (in_type == LCU_F32 && out_type == LCU_BF16) OUT(float, bf16_t);
+    else if (in_type == LCU_BF16 && out_type == LCU_BF16) OUT(bf16_t, bf16_t);
+    else return LCU_BAD_ARGUMENT;
+#undef OUT
+    LCU_LAUNCH_CHECK();
+    return LCU_OK;
+}

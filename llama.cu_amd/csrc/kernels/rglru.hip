@@ -1,0 +1,171 @@
+// The recurrent block with a real-gated linear recurrent unit.  The mixer's product gives, per token, two branches
+// of `width` channels, yin and xin (bias added here).  Then, per channel c and in 32-bit:
+//
+//   u   = conv_b + sum_j conv[c, j] * xin[t - taps + 1 + j]              (causal; rows before the request's start are zeros)
+//   r   = sigmoid(Wa[b] u_b + ba),  i = sigmoid(Wi[b] u_b + bi)          (the channels in `blocks` equal parts, a square matrix each)
+//   a   = exp(-c_exp * r * softplus(lam)),   S <- a * S + sqrt(1 - a^2) * i * u
+//   out = S * gelu_tanh(yin)
+//
+// Per request the state is [taps, width] floats: rows 0 .. taps-2 the last taps-1 rows of xin (oldest first), row
+// taps-1 the recurrence's S.  It is taken as zero where the request's first token of the step stands at position 0.
+// Three kernels: the convolution (a thread per token and channel), the gates (a workgroup per block of channels and
+// tile of tokens; the block's two matrices are given transposed, [block][in][out], so that the lanes read neighbours),
+// the scan (a thread per request and channel walks the request's tokens, then leaves the state).  sqrt(1 - a^2) is
+// taken as sqrt(-expm1(2 log a)): no cancellation where a is close to 1.
+#include "common.h"
+
+template <class TI>
+__global__ void rglru_conv_kernel(const TI *__restrict__ rows, int row_stride, int x_off, const float *__restrict__ bias,
+                                  const float *__restrict__ conv_w, const float *__restrict__ conv_b,
+                                  const float *__restrict__ state, float *__restrict__ u, const int *__restrict__ q_start,
+                                  const int *__restrict__ ctx_len, const int *__restrict__ req_of_token,
+                                  const int *__restrict__ state_slot, int width, int taps) {
+    const int t = blockIdx.x;
+    const int r = req_of_token[t];
+    const int t0 = q_start[r];
+    const int first_pos = ctx_len[r] - (q_start[r + 1] - t0);
+    const float *st = state + (size_t)state_slot[r] * taps * width;
+    for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < width; c += gridDim.y * blockDim.x) {
+        float acc = conv_b ? conv_b[c] : 0.f;
+        for (int j = 0; j < taps; ++j) {
+            const int back = taps - 1 - j;                       // how many tokens before t
+            float x = 0.f;
+            if (t - back >= t0) x = to_f32(rows[(size_t)(t - back) * row_stride + x_off + c]) + (bias ? bias[x_off + c] : 0.f);
+            else if (first_pos > 0) {
+                // the row that stood (t0 - (t - back)) tokens before the step: the state's last row is the newest
+                const int k = taps - 1 - (t0 - (t - back));
+                if (k >= 0 && first_pos - (t0 - (t - back)) >= 0) x = st[(size_t)k * width + c];
+            }
+            acc += conv_w[(size_t)c * taps + j] * x;
+        }
+        u[(size_t)t * width + c] = acc;
+    }
+}
+
+constexpr int RG_TOK = 8;          // tokens a workgroup of the gates kernel takes
+constexpr int RG_MAX_BS = 1024;    // channels of a block (LDS holds RG_TOK rows of them)
+
+__global__ void __launch_bounds__(256)
+rglru_gates_kernel(const float *__restrict__ u, const float *__restrict__ wa_t, const float *__restrict__ wi_t,
+                   const float *__restrict__ ba, const float *__restrict__ bi, const float *__restrict__ lam, float c_exp,
+                   float *__restrict__ a_out, float *__restrict__ gx_out, int n, int width, int bs) {
+    __shared__ float us[RG_TOK][RG_MAX_BS];
+    const int b = blockIdx.y, t0 = blockIdx.x * RG_TOK;
+    const int nt = min(RG_TOK, n - t0);
+    for (int w = threadIdx.x; w < RG_TOK * bs; w += blockDim.x) {
+        const int tt = w / bs, i = w % bs;
+        us[tt][i] = tt < nt ? u[(size_t)(t0 + tt) * width + b * bs + i] : 0.f;
+    }
+    __syncthreads();
+    const float *wa = wa_t + (size_t)b * bs * bs, *wi = wi_t + (size_t)b * bs * bs;
+    for (int o = threadIdx.x; o < bs; o += blockDim.x) {
+        float ra[RG_TOK], ri[RG_TOK];
+#pragma unroll
+        for (int tt = 0; tt < RG_TOK; ++tt) ra[tt] = ri[tt] = 0.f;
+        for (int i = 0; i < bs; ++i) {
+            const float a = wa[(size_t)i * bs + o], g = wi[(size_t)i * bs + o];
+#pragma unroll
+            for (int tt = 0; tt < RG_TOK; ++tt) {
+                ra[tt] += a * us[tt][i];
+                ri[tt] += g * us[tt][i];
+            }
+        }
+        const int c = b * bs + o;
+        const float l = lam[c];
+        const float sp = l > 20.f ? l : log1pf(expf(l));          // softplus
+        const float bias_a = ba[c], bias_i = bi[c];
+#pragma unroll
+        for (int tt = 0; tt < RG_TOK; ++tt) {
+            if (tt >= nt) break;
+            const float r = 1.0f / (1.0f + expf(-(ra[tt] + bias_a)));
+            const float gate = 1.0f / (1.0f + expf(-(ri[tt] + bias_i)));
+            const float log_a = -c_exp * r * sp;
+            const float mult = sqrtf(-expm1f(2.0f * log_a));
+            a_out[(size_t)(t0 + tt) * width + c] = expf(log_a);
+            gx_out[(size_t)(t0 + tt) * width + c] = mult * gate * us[tt][o];
+        }
+    }
+}
+
+__device__ __forceinline__ float gelu_tanh(float z) {
+    return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+}
+
+template <class TI, class T>
+__global__ void rglru_scan_kernel(const TI *__restrict__ rows, int row_stride, int y_off, int x_off, const float *__restrict__ bias,
+                                  const float *__restrict__ a, const float *__restrict__ gx, float *__restrict__ state,
+                                  T *__restrict__ out, const int *__restrict__ q_start, const int *__restrict__ ctx_len,
+                                  const int *__restrict__ state_slot, int width, int taps) {
+    const int r = blockIdx.y;
+    const int c = blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= width) return;
+    const int t0 = q_start[r], t1 = q_start[r + 1];
+    if (t1 <= t0) return;
+    const int first_pos = ctx_len[r] - (t1 - t0);
+    float *st = state + (size_t)state_slot[r] * taps * width;
+    float S = first_pos > 0 ? st[(size_t)(taps - 1) * width + c] : 0.f;
+    const float by = bias ? bias[y_off + c] : 0.f;
+    for (int t = t0; t < t1; ++t) {
+        S = a[(size_t)t * width + c] * S + gx[(size_t)t * width + c];
+        const float y = gelu_tanh(to_f32(rows[(size_t)t * row_stride + y_off + c]) + by);
+        out[(size_t)t * width + c] = from_f32<T>(S * y);
+    }
+    st[(size_t)(taps - 1) * width + c] = S;
+    // the convolution's state: the last taps - 1 rows of xin, oldest first; where the step brought fewer, older rows move up
+    const int q = t1 - t0;
+    const float bx = bias ? bias[x_off + c] : 0.f;
+    float keep[16];
+    for (int k = 0; k < taps - 1; ++k) {
+        const int back = taps - 1 - k;                           // row k is the one `back` tokens before the request's end
+        float x = 0.f;
+        if (back <= q) x = to_f32(rows[(size_t)(t1 - back) * row_stride + x_off + c]) + bx;
+        else if (first_pos > 0) {
+            const int old = k + q;                               // where that row stands in the state as the step found it
+            if (old < taps - 1 && first_pos - (back - q) >= 0) x = st[(size_t)old * width + c];
+        }
+        keep[k] = x;
+    }
+    for (int k = 0; k < taps - 1; ++k) st[(size_t)k * width + c] = keep[k];
+}
+
+// rows: [n, row_stride] of in_type, yin at y_off and xin at x_off (width each); bias: null or float32 over the row's
+// columns.  conv_w [width, taps], conv_b [width] (may be null), wa_t / wi_t [blocks, bs, bs] transposed ([in][out]),
+// ba / bi / lam [width], all float32.  state: float32 [slots, taps, width].  u, a, gx: float32 scratch [n, width].
+// out: [n, width] of out_type.
+LCU_API int lcu_rglru(const void *rows, int in_type, int row_stride, int y_off, int x_off, const float *bias,
+                      const float *conv_w, const float *conv_b, const float *wa_t, const float *wi_t, const float *ba,
+                      const float *bi, const float *lam, float c_exp, float *state, float *u, float *a, float *gx, void *out,
+                      int out_type, const int *q_start, const int *ctx_len, const int *req_of_token, const int *state_slot,
+                      int n, int n_req, int width, int blocks, int taps, hipStream_t stream) {
+    if (n <= 0 || n_req <= 0) return LCU_OK;
+    if (width <= 0 || blocks <= 0 || width % blocks || width / blocks > RG_MAX_BS || taps < 1 || taps > 16 || n_req > 65535 ||
+        !rows || !conv_w || !wa_t || !wi_t || !ba || !bi || !lam || !state || !u || !a || !gx || !out)
+        return LCU_BAD_ARGUMENT;
+    const int bs = width / blocks;
+    {
+        dim3 grid(n, (width + 1023) / 1024 > 0 ? (width + 1023) / 1024 : 1), block(256);
+        if (in_type == LCU_F32)
+            rglru_conv_kernel<float><<<grid, block, 0, stream>>>((const float *)rows, row_stride, x_off, bias, conv_w, conv_b, state, u, q_start, ctx_len, req_of_token, state_slot, width, taps);
+        else if (in_type == LCU_BF16)
+            rglru_conv_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t *)rows, row_stride, x_off, bias, conv_w, conv_b, state, u, q_start, ctx_len, req_of_token, state_slot, width, taps);
+        else
+            return LCU_BAD_ARGUMENT;
+        LCU_LAUNCH_CHECK();
+    }
+    {
+        dim3 grid((n + RG_TOK - 1) / RG_TOK, blocks), block(bs >= 256 ? 256 : (bs + 63) / 64 * 64);
+        rglru_gates_kernel<<<grid, block, 0, stream>>>(u, wa_t, wi_t, ba, bi, lam, c_exp, a, gx, n, width, bs);
+        LCU_LAUNCH_CHECK();
+    }
+    {
+        dim3 grid((width + 63) / 64, n_req), block(64);
+#define GO(TI, T) rglru_scan_kernel<TI, T><<<grid, block, 0, stream>>>((const TI *)rows, row_stride, y_off, x_off, bias, a, gx, state, (T *)out, q_start, ctx_len, state_slot, width, taps)
+        if (in_type == LCU_F32 && out_type == LCU_F32) GO(float, float);
+        else if (in_type == LCU_F32 && out_type == LCU_BF16) GO(float, bf16_t);
+        else if (in_type == LCU_BF16 && out_type == LCU_BF16) GO(bf16_t, bf16_t);
+        else return LCU_BAD_ARGUMENT;
+#undef GO
+        LCU_LAUNCH_CHECK();
+    }
+    return LCU_OK;
+}

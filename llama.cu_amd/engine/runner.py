@@ -164,7 +164,7 @@ class ModelRunner:
                     made = need.allocate(group, pages, ps, self.max_seqs, self.dtype, self.device)
                 self.caches.append(made)
         for made, states in zip(self.caches, own_states):       # what each entry's block keeps itself, per request
-            made.more = {name: s.allocate(-1, 0, 0, self.max_seqs, self.dtype, self.device).state for name, s in states.items()}
+            made.more.update({name: s.allocate(-1, 0, 0, self.max_seqs, self.dtype, self.device).state for name, s in states.items()})
         max_pages = [(self.max_model_len + g.page_size - 1) // g.page_size for g in self.groups]
         self.builder = BatchBuilder(self.cache, self.max_batch_tokens, self.max_seqs, max_pages, self.device)
         # a debugging aid: pages that were given back, or went to another request, since the last step are

@@ -36,7 +36,8 @@ HOST_FLAGS = ["-O2", "-std=c++17", "-shared", "-fPIC", "-Wall", "-pthread", "-ff
 HIP_FLAGS += os.environ.get("LCU_HIP_FLAGS", "").split()
 
 KERNEL_LIBRARIES = ["elementwise", "rope_kv", "attention_generic", "attention_mfma", "attention_mfma_bias", "gemm_generic", "gemm_skinny",
-                    "gemm_mid", "sampling", "random_fill", "norm_conv", "qk_norm", "delta_rule", "moe"]
+                    "gemm_mid", "sampling", "random_fill", "norm_conv", "qk_norm", "delta_rule", "moe", "norm_post", "qkv_prepare",
+                    "retention", "rglru"]
 HOST_LIBRARY = "host"
 
 _loaded: Dict[str, ctypes.CDLL] = {}

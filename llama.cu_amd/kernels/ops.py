@@ -312,10 +312,12 @@ def _attention_args(q, out, cache, block_table, q_start, ctx_len, req_of_token, 
 def paged_attention_generic(q: torch.Tensor, out: torch.Tensor, cache: torch.Tensor, block_table: torch.Tensor,
                             q_start: torch.Tensor, ctx_len: torch.Tensor, req_of_token: torch.Tensor,
                             n_heads: int, n_kv_heads: int, head_dim: int, page_size: int, scale: float,
-                            window: int = 0, head_slopes: Optional[torch.Tensor] = None, value_dim: int = 0) -> torch.Tensor:
+                            window: int = 0, head_slopes: Optional[torch.Tensor] = None, value_dim: int = 0,
+                            chunk: int = 0) -> torch.Tensor:
     """Causal attention of the step's queries over the paged cache (every shape).  ``head_slopes``
     (float32 [n_heads]) adds ``slope[h] * (key position - query position)`` to the scaled scores.
-    ``value_dim``: the values' head size if it is not the keys' (``out`` is ``[n, n_heads * value_dim]``)."""
+    ``value_dim``: the values' head size if it is not the keys' (``out`` is ``[n, n_heads * value_dim]``).
+    ``chunk``: the query at position ``p`` sees the keys from ``p - p % chunk`` on only (instead of a window)."""
     n = _attention_args(q, out, cache, block_table, q_start, ctx_len, req_of_token, n_heads, n_kv_heads, head_dim,
                         page_size, value_dim)
     value_dim = value_dim or head_dim
@@ -329,7 +331,8 @@ def paged_attention_generic(q: torch.Tensor, out: torch.Tensor, cache: torch.Ten
     _check(lib.lcu_paged_attention_generic(_ptr(q), q.stride(0), _ptr(out), out.stride(0), _type(q, "q"), _ptr(cache),
                                            _ptr(block_table), block_table.shape[1], _ptr(q_start), _ptr(ctx_len),
                                            _ptr(req_of_token), n, n_heads, n_kv_heads, head_dim, value_dim, page_size,
-                                           ctypes.c_float(scale), int(window), _ptr(head_slopes), _stream()), "paged_attention_generic")
+                                           ctypes.c_float(scale), int(window), int(chunk), _ptr(head_slopes), _stream()),
+           "paged_attention_generic")
     return out
 
 
@@ -554,19 +557,21 @@ def decode_splits(n_req: int, n_heads: int, n_kv_heads: int, max_ctx_len: int) -
 
 def paged_attention(q: torch.Tensor, out: torch.Tensor, cache: torch.Tensor, step, group: int, n_heads: int,
                     n_kv_heads: int, head_dim: int, page_size: int, scale: float, window: int = 0,
-                    force_generic: bool = False, head_slopes: Optional[torch.Tensor] = None, value_dim: int = 0) -> torch.Tensor:
+                    force_generic: bool = False, head_slopes: Optional[torch.Tensor] = None, value_dim: int = 0,
+                    chunk: int = 0) -> torch.Tensor:
     """Attention for the batch ``step`` (an engine.batch.StepContext) over cache group
-    ``group``: picks the kernel for the batch's shape and type.  With a bias inside the scores
+    ``group``: picks the kernel for the batch's shape and type.  ``chunk``: keys of the query's own chunk of so many
+    positions only (the generic kernel).  With a bias inside the scores
     (``head_slopes``) the matrix-core kernels are those of the second library, which need a positive scale."""
     bt = step.block_table(group)
     if head_slopes is not None:
         _gpu(head_slopes)
         if head_slopes.dtype != torch.float32 or head_slopes.shape != (n_heads,) or not head_slopes.is_contiguous():
             raise KernelError(f"attention: head_slopes must be contiguous float32 [{n_heads}]")
-    if force_generic or (head_slopes is not None and not scale > 0) or (value_dim and value_dim != head_dim) \
+    if force_generic or chunk or (head_slopes is not None and not scale > 0) or (value_dim and value_dim != head_dim) \
             or not mfma_attention_supported(q, n_heads, n_kv_heads, head_dim, page_size):
         return paged_attention_generic(q, out, cache, bt, step.q_start, step.ctx_len, step.req_of_token, n_heads,
-                                       n_kv_heads, head_dim, page_size, scale, window, head_slopes, value_dim)
+                                       n_kv_heads, head_dim, page_size, scale, window, head_slopes, value_dim, chunk)
     n = _attention_args(q, out, cache, bt, step.q_start, step.ctx_len, step.req_of_token, n_heads, n_kv_heads, head_dim,
                         page_size)
     if step.decode_only:
@@ -1198,4 +1203,193 @@ def moe_experts(h: torch.Tensor, ids: torch.Tensor, wts: torch.Tensor, w_up: tor
     y = torch.empty((total, d), dtype=torch.float32, device=h.device) if top > 1 else None
     _check(lib.lcu_moe_experts(_ptr(h), _type(h, "moe input"), _ptr(ids), _ptr(wts), _ptr(ints), max_tiles, _ptr(w_up),
                                _ptr(w_down), _ptr(act), _ptr(y), _ptr(out), n, d, ff, experts, top, _stream()), "moe_experts")
+    return out
+
+
+# ------------------------------------------------------------------ norms behind a sublayer
+
+
+def norm_post(x: torch.Tensor, a: torch.Tensor, w_post: torch.Tensor, eps_post: float, w_pre: Optional[torch.Tensor] = None,
+              eps_pre: float = 0.0, out_dtype: Optional[torch.dtype] = None) -> Optional[torch.Tensor]:
+    """``x += a * rsqrt(mean(a^2) + eps_post) * w_post`` (``x``: the float32 residual stream, in place; ``a``: a
+    sublayer's output) and, with ``w_pre``, the rows ``x * rsqrt(mean(x^2) + eps_pre) * w_pre`` of the norm that
+    follows, in ``out_dtype``; one kernel.  The weights are float32 factors."""
+    _gpu(x, a, w_post, w_pre)
+    _rows(x, "residual stream"); _contig(x, "residual stream"); _contig(a, "sublayer output")
+    n, d = x.shape
+    if x.dtype != torch.float32 or a.shape != (n, d):
+        raise KernelError(f"norm_post: the stream must be float32 and the sublayer's output of its shape, got {x.dtype} {tuple(x.shape)} and {tuple(a.shape)}")
+    _f32_vec(w_post, "norm weight", d); _f32_vec(w_pre, "norm weight", d)
+    out = None
+    if w_pre is not None:
+        out = torch.empty((n, d), dtype=out_dtype or a.dtype, device=x.device)
+    lib = build.load("norm_post")
+    _check(lib.lcu_norm_post(_ptr(x), _ptr(a), _type(a, "sublayer output"), _ptr(w_post), ctypes.c_float(eps_post), _ptr(w_pre),
+                             ctypes.c_float(eps_pre), _ptr(out), _type(out, "norm out") if out is not None else F32, n, d,
+                             _stream()), "norm_post")
+    return out
+
+
+def scaled_sum(acc: Optional[torch.Tensor], x: torch.Tensor, scale: float) -> torch.Tensor:
+    """``acc + scale * x`` in 32-bit, in place in ``acc`` (float32); ``acc=None`` starts a new sum of ``x``'s shape."""
+    _gpu(acc, x)
+    _contig(x, "scaled_sum x")
+    first = acc is None
+    if first:
+        acc = torch.empty(x.shape, dtype=torch.float32, device=x.device)
+    _contig(acc, "scaled_sum acc")
+    if acc.dtype != torch.float32 or acc.shape != x.shape:
+        raise KernelError("scaled_sum: the sum must be float32 and of the addend's shape")
+    lib = build.load("norm_post")
+    _check(lib.lcu_scaled_sum(_ptr(acc), _ptr(x), _type(x, "scaled_sum x"), ctypes.c_float(scale), ctypes.c_longlong(x.numel()),
+                              int(first), _stream()), "scaled_sum")
+    return acc
+
+
+# ------------------------------------------------------------------ bias, head norm, rotation, cache write
+
+
+def qkv_prepare(rows: torch.Tensor, offsets, n_heads: int, n_kv_heads: int, head_dim: int, value_dim: int, stored_dim: int,
+                stored_value_dim: int, dtype: torch.dtype, positions: Optional[torch.Tensor] = None,
+                bias: Optional[torch.Tensor] = None, q_norm: Optional[torch.Tensor] = None, k_norm: Optional[torch.Tensor] = None,
+                eps: float = 0.0, cos: Optional[torch.Tensor] = None, sin: Optional[torch.Tensor] = None, rot_dim: int = 0,
+                pairing: int = 0, cache: Optional[torch.Tensor] = None, slots: Optional[torch.Tensor] = None,
+                page_size: int = 16) -> torch.Tensor:
+    """What stands between a q, k, v product and its attention, each piece optional: ``rows [n, *]`` holds the product
+    with q at column ``offsets[0]`` (``n_heads * head_dim``), k at ``offsets[1]``, v at ``offsets[2]`` (``n_kv_heads *
+    value_dim``); ``bias`` (float32 over the rows' columns) is added; q and k are divided by the root mean square over
+    each head and multiplied by ``q_norm`` / ``k_norm`` (float32 ``[head_dim]``); the first ``rot_dim`` dims of every q and
+    k head are rotated (tables ``cos``, ``sin``; ``pairing`` 0: halves, 1: neighbours).  Returns q as ``[n, n_heads *
+    stored_dim]`` of ``dtype`` and writes k and v into ``cache`` at ``slots`` with ``stored_dim`` / ``stored_value_dim`` dims
+    a head, the dims beyond the true ones zeros.  ``cache=None``: queries only."""
+    _gpu(rows, positions, bias, q_norm, k_norm, cos, sin, cache, slots)
+    _rows(rows, "qkv rows")
+    n, width = rows.shape
+    store = cache is not None
+    q_off, k_off, v_off = (int(o) for o in offsets)
+    if q_off < 0 or q_off + n_heads * head_dim > width or (store and (k_off < 0 or k_off + n_kv_heads * head_dim > width
+                                                                      or v_off < 0 or v_off + n_kv_heads * value_dim > width)):
+        raise KernelError(f"qkv_prepare: the columns of q, k or v lie outside the rows' {width} columns")
+    if stored_dim % 8 or stored_dim < head_dim or stored_value_dim < value_dim or max(stored_dim, stored_value_dim) > 256:
+        raise KernelError(f"qkv_prepare: stored head sizes {stored_dim} / {stored_value_dim} do not fit {head_dim} / {value_dim} (keys a multiple of 8, at most 256)")
+    _f32_vec(bias, "qkv bias", width); _f32_vec(q_norm, "query norm weight", head_dim); _f32_vec(k_norm, "key norm weight", head_dim)
+    max_pos = 0
+    if cos is not None:
+        if sin is None or cos.shape != sin.shape or cos.dtype != torch.float32 or sin.dtype != torch.float32 or positions is None \
+                or cos.dim() != 2 or cos.shape[1] * 2 != rot_dim or not cos.is_contiguous() or not sin.is_contiguous():
+            raise KernelError("rotation tables must be two contiguous float32 tensors [max_pos, rot_dim/2], with the positions")
+        _i32(positions, "positions", n)
+        max_pos = cos.shape[0]
+    if store:
+        _i32(slots, "cache slots", n)
+        _contig(cache, "cache")
+        if cache.dtype != dtype or cache.dim() != 3 or cache.shape[1] * cache.shape[2] != n_kv_heads * (stored_dim + stored_value_dim) * page_size:
+            raise KernelError(f"cache: {cache.dtype} {tuple(cache.shape)} does not hold pages of {n_kv_heads} x ({stored_dim} + {stored_value_dim}) x {page_size} {dtype}")
+    q = torch.empty((n, n_heads * stored_dim), dtype=dtype, device=rows.device)
+    lib = build.load("qkv_prepare")
+    _check(lib.lcu_qkv_prepare(_ptr(rows), _type(rows, "qkv rows"), n, rows.stride(0), q_off, k_off, v_off, _ptr(bias), _ptr(q_norm),
+                               _ptr(k_norm), ctypes.c_float(eps), _ptr(positions), _ptr(cos), _ptr(sin), max_pos, int(rot_dim), int(pairing),
+                               _ptr(q), _type(q, "q"), _ptr(slots), _ptr(cache), n_heads, n_kv_heads if store else 0, head_dim,
+                               stored_dim, value_dim, stored_value_dim, page_size, int(store), _stream()), "qkv_prepare")
+    return q
+
+
+def head_gate(out: torch.Tensor, gate_rows: torch.Tensor, g_off: int, n_heads: int, value_dim: int) -> torch.Tensor:
+    """``out[t, h, :] *= sigmoid(gate_rows[t, g_off + h])`` for ``out [n, n_heads * value_dim]``, in place."""
+    _gpu(out, gate_rows)
+    _rows(out, "attention out"); _contig(out, "attention out"); _rows(gate_rows, "gate rows")
+    n = out.shape[0]
+    if out.shape[1] != n_heads * value_dim or gate_rows.shape[0] != n or g_off < 0 or g_off + n_heads > gate_rows.shape[1]:
+        raise KernelError("head_gate: the output or the gates' columns do not fit")
+    lib = build.load("qkv_prepare")
+    _check(lib.lcu_head_gate(_ptr(out), _type(out, "attention out"), _ptr(gate_rows), _type(gate_rows, "gate rows"),
+                             gate_rows.stride(0), int(g_off), n, n_heads, value_dim, _stream()), "head_gate")
+    return out
+
+
+# ------------------------------------------------------------------ retention
+
+
+def retention(rows: torch.Tensor, offsets: Dict[str, int], decay: torch.Tensor, state: torch.Tensor, step, heads: int,
+              key_dim: int, value_dim: int, k_scale: float, eps: float, out_dtype: torch.dtype,
+              cos: Optional[torch.Tensor] = None, sin: Optional[torch.Tensor] = None, rot_dim: int = 0, pairing: int = 0) -> torch.Tensor:
+    """Linear attention with a fixed decay per head over the step's rows, request by request from each request's state
+    (``state [slots, heads, key_dim, value_dim]`` float32, taken as zero at a request's position 0 and left as the
+    step's last token makes it): ``S <- decay[h] S + k v^T``, ``o = S^T q``.  ``rows [n, *]`` holds q, k (``heads *
+    key_dim``), v and the gate g (``heads * value_dim``) at the columns ``offsets``; q and k are rotated (tables, as
+    ``qkv_prepare``), k then multiplied by ``k_scale``.  Returns each head's ``o`` divided by its root mean square
+    (``eps``) times ``silu(g)``, ``[n, heads * value_dim]`` in ``out_dtype``."""
+    _gpu(rows, decay, state, cos, sin)
+    _rows(rows, "retention rows")
+    n, width = rows.shape
+    hk, hv = heads * key_dim, heads * value_dim
+    for name, w in (("q", hk), ("k", hk), ("v", hv), ("g", hv)):
+        if name not in offsets or offsets[name] < 0 or offsets[name] + w > width:
+            raise KernelError(f"retention: the columns of {name!r} lie outside the rows' {width} columns")
+    _f32_vec(decay, "retention decay", heads)
+    if key_dim > 256:
+        raise KernelError(f"retention: key size {key_dim} is not supported (at most 256)")
+    if state.dtype != torch.float32 or not state.is_contiguous() or state.dim() != 4 or state.shape[1:] != (heads, key_dim, value_dim):
+        raise KernelError(f"retention: state must be contiguous float32 [slots, {heads}, {key_dim}, {value_dim}]")
+    if n != step.n or max(step.state_slots, default=0) >= state.shape[0]:
+        raise KernelError("retention: the rows are not the step's, or a request's slot lies outside the state")
+    max_pos = 0
+    if cos is not None:
+        if sin is None or cos.shape != sin.shape or cos.dtype != torch.float32 or sin.dtype != torch.float32 \
+                or cos.dim() != 2 or cos.shape[1] * 2 != rot_dim or not cos.is_contiguous() or not sin.is_contiguous():
+            raise KernelError("rotation tables must be two contiguous float32 tensors [max_pos, rot_dim/2]")
+        max_pos = cos.shape[0]
+    o = torch.empty((n, hv), dtype=torch.float32, device=rows.device)
+    out = torch.empty((n, hv), dtype=out_dtype, device=rows.device)
+    lib = build.load("retention")
+    _check(lib.lcu_retention(_ptr(rows), _type(rows, "retention rows"), rows.stride(0), offsets["q"], offsets["k"], offsets["v"],
+                             offsets["g"], _ptr(step.positions), _ptr(cos), _ptr(sin), max_pos, int(rot_dim), int(pairing),
+                             ctypes.c_float(k_scale), _ptr(decay), _ptr(state), _ptr(o), _ptr(out), _type(out, "retention out"),
+                             _ptr(step.q_start), _ptr(step.ctx_len), _ptr(step.state_slot), n, step.n_req, heads, key_dim,
+                             value_dim, ctypes.c_float(eps), _stream()), "retention")
+    return out
+
+
+# ------------------------------------------------------------------ the gated linear recurrent unit
+
+
+def rglru(rows: torch.Tensor, y_off: int, x_off: int, bias: Optional[torch.Tensor], conv_w: torch.Tensor,
+          conv_b: Optional[torch.Tensor], wa_t: torch.Tensor, wi_t: torch.Tensor, ba: torch.Tensor, bi: torch.Tensor,
+          lam: torch.Tensor, c_exp: float, state: torch.Tensor, step, out_dtype: torch.dtype) -> torch.Tensor:
+    """The recurrent block between its input product and its output product.  ``rows [n, *]`` holds the two branches
+    (``width`` columns each at ``y_off`` and ``x_off``; ``bias`` float32 over the rows' columns is added).  ``u`` = causal
+    convolution of the x branch (``conv_w [width, taps]``, the last column the current token's; ``conv_b``); gates ``r =
+    sigmoid(Wa u + ba)``, ``i = sigmoid(Wi u + bi)`` with block-diagonal matrices given transposed (``wa_t``, ``wi_t``
+    ``[blocks, in, out]``); ``a = exp(-c_exp r softplus(lam))``; ``S <- a S + sqrt(1 - a^2) i u``; returns ``S *
+    gelu_tanh(y branch)`` as ``[n, width]`` in ``out_dtype``.  ``state [slots, taps, width]`` float32: the last ``taps -
+    1`` rows of the x branch, then ``S``; taken as zero at a request's position 0."""
+    _gpu(rows, bias, conv_w, conv_b, wa_t, wi_t, ba, bi, lam, state)
+    _rows(rows, "rglru rows")
+    n, cols = rows.shape
+    if conv_w.dim() != 2 or conv_w.dtype != torch.float32 or not conv_w.is_contiguous():
+        raise KernelError("rglru: the convolution's weight must be contiguous float32 [width, taps]")
+    width, taps = conv_w.shape
+    if wa_t.dim() != 3 or wa_t.shape != wi_t.shape or wa_t.shape[1] != wa_t.shape[2] or wa_t.shape[0] * wa_t.shape[1] != width \
+            or wa_t.dtype != torch.float32 or wi_t.dtype != torch.float32 or not wa_t.is_contiguous() or not wi_t.is_contiguous():
+        raise KernelError(f"rglru: the gates' matrices must be contiguous float32 [blocks, width / blocks, width / blocks] for width {width}")
+    blocks = wa_t.shape[0]
+    if width // blocks > 1024 or taps > 16:
+        raise KernelError(f"rglru: blocks of {width // blocks} channels or {taps} taps are not supported (at most 1024 and 16)")
+    for name, off in (("y", y_off), ("x", x_off)):
+        if off < 0 or off + width > cols:
+            raise KernelError(f"rglru: the columns of the {name} branch lie outside the rows' {cols} columns")
+    _f32_vec(bias, "rglru bias", cols); _f32_vec(conv_b, "rglru conv bias", width)
+    _f32_vec(ba, "rglru gate bias", width); _f32_vec(bi, "rglru gate bias", width); _f32_vec(lam, "rglru lam", width)
+    if state.dtype != torch.float32 or not state.is_contiguous() or state.dim() != 3 or state.shape[1:] != (taps, width):
+        raise KernelError(f"rglru: state must be contiguous float32 [slots, {taps}, {width}]")
+    if n != step.n or max(step.state_slots, default=0) >= state.shape[0]:
+        raise KernelError("rglru: the rows are not the step's, or a request's slot lies outside the state")
+    scratch = torch.empty((3, n, width), dtype=torch.float32, device=rows.device)
+    out = torch.empty((n, width), dtype=out_dtype, device=rows.device)
+    lib = build.load("rglru")
+    _check(lib.lcu_rglru(_ptr(rows), _type(rows, "rglru rows"), rows.stride(0), int(y_off), int(x_off), _ptr(bias), _ptr(conv_w),
+                         _ptr(conv_b), _ptr(wa_t), _ptr(wi_t), _ptr(ba), _ptr(bi), _ptr(lam), ctypes.c_float(c_exp), _ptr(state),
+                         _ptr(scratch[0]), _ptr(scratch[1]), _ptr(scratch[2]), _ptr(out), _type(out, "rglru out"), _ptr(step.q_start),
+                         _ptr(step.ctx_len), _ptr(step.req_of_token), _ptr(step.state_slot), n, step.n_req, width, blocks, taps,
+                         _stream()), "rglru")
     return out

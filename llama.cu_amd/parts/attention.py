@@ -24,13 +24,23 @@ class Attention(Part):
 
     # the tensors' names under the part's own, as files with config.json's names hold them; ``names`` replaces any
     NAMES = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight",
-             "q_norm": "q_norm.weight", "k_norm": "k_norm.weight"}
+             "q_norm": "q_norm.weight", "k_norm": "k_norm.weight", "q_bias": "q_proj.bias", "k_bias": "k_proj.bias",
+             "v_bias": "v_proj.bias", "q_head_norm": "q_head_norm.weight", "k_head_norm": "k_head_norm.weight", "g": "g_proj.weight"}
 
     def __init__(self, hidden_size: int, heads: int, kv_heads: int, head_dim: int, scale: Optional[float] = None,
                  window: int = 0, position: Optional[PartSpec] = None, shares_kv: bool = False, page_size: int = 0,
                  value_dim: int = 0, projection_norm_eps: Optional[float] = None, query_temperature=None,
-                 names: Optional[Dict[str, str]] = None):
-        """``value_dim``: the values' head size if it is not ``head_dim``.  ``projection_norm_eps``: queries and keys
+                 names: Optional[Dict[str, str]] = None, bias: bool = False, head_norm_eps: Optional[float] = None,
+                 chunk: int = 0, head_gate: bool = False):
+        """``bias``: q, k and v have biases (tensors ``q_bias``, ``k_bias``, ``v_bias``), added in the projection.
+        ``head_norm_eps``: every q and k head is divided by its root mean square and multiplied by a weight over the
+        head's dims that all heads share (tensors ``q_head_norm``, ``k_head_norm``), before any rotation.  ``chunk``: the
+        query at position ``p`` sees only the keys from ``p - p % chunk`` on (instead of a window).  ``head_gate``: each
+        head's output is multiplied by the sigmoid of a number that a projection of the mixer's input gives for the
+        head (tensor ``g`` ``[heads, hidden]``).  With any of these, with values of another head size than the keys'
+        under a rotation, or with a rotation of a part of a head whose size is no multiple of 8, the mixer runs its
+        general path: one product for all projections with 32-bit output, then ``ops.qkv_prepare``.
+        ``value_dim``: the values' head size if it is not ``head_dim``.  ``projection_norm_eps``: queries and keys
         are divided by the root mean square over their whole projection (all heads at once) and multiplied by a
         weight per column (tensors ``q_norm``, ``k_norm``).  ``query_temperature = (coef, every)``: the query at
         position ``p`` is multiplied by ``1 + coef * ln(floor((p + 1) / every) + 1)``."""
@@ -52,6 +62,11 @@ class Attention(Part):
                 raise ValueError(f"attention: the query temperature's step {every} must be at least 1")
             self.q_temp = (float(coef), int(every))
         self.names = dict(self.NAMES, **(names or {}))
+        self.bias, self.head_gate = bool(bias), bool(head_gate)
+        self.head_norm_eps = None if head_norm_eps is None else float(head_norm_eps)
+        self.chunk = int(chunk or 0)
+        if self.chunk and self.window:
+            raise ValueError("attention: a window and chunks together are not supported")
         # the kernels read keys eight dims at a time: a head size that is no multiple of 8 is filled up with dims of
         # zeros (rows of zeros in the q and k matrices), which change no score; only without a rotation, whose pairs
         # would not know of them
@@ -61,6 +76,14 @@ class Attention(Part):
         self.shares_kv = bool(shares_kv)          # reads another layer's keys and values: has q and o only
         self.position = make_part("position", position or PartSpec("none"))
         self.graph_safe = self.position.graph_safe
+        rot = self.position.rotated_dims()
+        self.general = bool(self.bias or self.head_gate or self.head_norm_eps is not None or self.chunk
+                            or (rot and (self.value_dim != self.head_dim or self.padded_dim != self.head_dim)))
+        if self.general and (self.shares_kv or self.norm_eps is not None or self.q_temp is not None):
+            raise ValueError("attention: biases, head norms, chunks, a head gate or values of their own size under a rotation "
+                             "do not go together with shared keys and values, a norm over the whole projection or a query temperature")
+        # what a head takes in the cache and in the kernels: the true sizes filled up with dims of zeros (general path)
+        self.stored_dim, self.stored_value_dim = self.padded_dim, self.value_dim
         self.w_qkv = self.w_o = None
         self.page_size = 0
 
@@ -74,14 +97,29 @@ class Attention(Part):
             t[nm["q_norm"]] = TensorSpec((nh * dh,), init="one_plus_normal")
             if not self.shares_kv:
                 t[nm["k_norm"]] = TensorSpec((nkv * dh,), init="one_plus_normal")
+        if self.bias:
+            t[nm["q_bias"]] = TensorSpec((nh * dh,))
+            t[nm["k_bias"]] = TensorSpec((nkv * dh,))
+            t[nm["v_bias"]] = TensorSpec((nkv * dv,))
+        if self.head_norm_eps is not None:
+            t[nm["q_head_norm"]] = TensorSpec((dh,), init="one_plus_normal")
+            t[nm["k_head_norm"]] = TensorSpec((dh,), init="one_plus_normal")
+        if self.head_gate:
+            t[nm["g"]] = TensorSpec((nh, d))
         return t
 
     def fused_groups(self, dtype, device):
+        if self.general:
+            return [(tuple(self.names[k] for k in ("q", "k", "v") + (("g",) if self.head_gate else ())), 0)]
         if self.shares_kv or self.padded_dim != self.head_dim:
             return []
         return [((self.names["q"], self.names["k"], self.names["v"]), 0)]
 
     def cache_need(self):
+        if self.general:
+            # (a chunk's pages are given back like a window's: no query looks further back than a chunk's length)
+            return PagedKV(self.kv_heads, self.stored_dim, self.window or self.chunk, self.own_page_size,
+                           self.stored_value_dim if self.stored_value_dim != self.stored_dim else 0)
         return PagedKV(self.kv_heads, self.padded_dim, self.window, self.own_page_size,
                        self.value_dim if self.value_dim != self.padded_dim else 0)
 
@@ -99,7 +137,51 @@ class Attention(Part):
         requests decode over at most ``max_ctx_len`` keys (a captured graph fixes the number)."""
         return ops.decode_splits(batch, self.heads, self.kv_heads, max_ctx_len)
 
+    def _load_general(self, tensors, build: BuildContext) -> None:
+        nm, nh, nkv, dh, dv = self.names, self.heads, self.kv_heads, self.head_dim, self.value_dim
+        mats = [tensors[nm["q"]], tensors[nm["k"]], tensors[nm["v"]]] + ([tensors[nm["g"]]] if self.head_gate else [])
+        self.w_in = Weight(fused_rows(mats), build)
+        self.offsets = (0, nh * dh, (nh + nkv) * dh)
+        self.g_off = (nh + nkv) * dh + nkv * dv
+        self.bias_vec = None
+        if self.bias:       # one vector over the product's columns, 32-bit: added before anything is rounded
+            parts = [tensors[nm[k]].float() for k in ("q_bias", "k_bias", "v_bias")]
+            if self.head_gate:
+                parts.append(torch.zeros(nh, dtype=torch.float32, device=parts[0].device))
+            self.bias_vec = torch.cat(parts).contiguous()
+        self.q_head_norm = self.k_head_norm = None
+        if self.head_norm_eps is not None:
+            self.q_head_norm = tensors[nm["q_head_norm"]].float().contiguous()
+            self.k_head_norm = tensors[nm["k_head_norm"]].float().contiguous()
+        self.w_o = Weight(tensors[nm["o"]], build)
+        self.position.load({}, build)
+        if type(self.position).apply is not Part.apply or self.position.score_slopes() is not None:
+            raise ValueError("attention: the general path takes a rotation or no position encoding")
+        self.page_size = build.page_size
+        self.dtype = build.dtype
+
+    def _forward_general(self, h, step, cache, out_dtype=None):
+        nh, nkv = self.heads, self.kv_heads
+        if not cache.writes:
+            raise ops.KernelError("attention: the general path needs a cache of its own")
+        page_size = cache.page_size or self.page_size
+        rot = self.position.rotary_tables()
+        cos, sin, rot_dim, pairing = rot if rot is not None else (None, None, 0, 0)
+        rows = linear(h, self.w_in, out_dtype=torch.float32)
+        q = ops.qkv_prepare(rows, self.offsets, nh, nkv, self.head_dim, self.value_dim, self.stored_dim, self.stored_value_dim,
+                            self.dtype, positions=step.positions, bias=self.bias_vec, q_norm=self.q_head_norm,
+                            k_norm=self.k_head_norm, eps=self.head_norm_eps or 0.0, cos=cos, sin=sin, rot_dim=rot_dim,
+                            pairing=pairing, cache=cache.pages, slots=step.slots(cache.group), page_size=page_size)
+        out = torch.empty((rows.shape[0], nh * self.stored_value_dim), dtype=self.dtype, device=rows.device)
+        ops.paged_attention(q, out, cache.pages, step, cache.group, nh, nkv, self.stored_dim, page_size, self.scale,
+                            self.window, value_dim=self.stored_value_dim, chunk=self.chunk)
+        if self.head_gate:
+            ops.head_gate(out, rows, self.g_off, nh, self.stored_value_dim)
+        return linear(out, self.w_o, out_dtype=out_dtype or self.dtype)
+
     def load(self, tensors, build: BuildContext) -> None:
+        if self.general:
+            return self._load_general(tensors, build)
         nm = self.names
         if self.padded_dim != self.head_dim and self.position.rotary_tables() is not None:
             raise ValueError(f"attention: head_dim {self.head_dim} is no multiple of 8, which the kernels take only without a rotation")
@@ -136,6 +218,8 @@ class Attention(Part):
         """The lists by which the matrix-core kernels share out a step that is not all single tokens are made here, on
         the host, and go to the device with the step's arrays; ``forward`` then launches work whose sizes follow from
         the step's sizes alone."""
+        if self.general:
+            return
         page_size = self.own_page_size or self.page_size
         if self.dtype == torch.bfloat16 and (self.position.score_slopes() is None or self.scale > 0) \
                 and self.value_dim == self.padded_dim and ops.mfma_attention_refusal(self.dtype, self.heads, self.kv_heads, self.padded_dim, page_size) is None:
@@ -151,11 +235,15 @@ class Attention(Part):
         """Whether ``forward`` could be given ScaledRows of ``n_rows`` rows in the place of
         plain rows: only where the kernel for few rows is the faster one for the q, k, v
         product anyway."""
+        if self.general:
+            return False
         return self.dtype == torch.bfloat16 and n_rows <= ops.ADD_NORM_MAX_ROWS and skinny_takes(n_rows, self.w_qkv, preferred=True)
 
     def forward(self, h, step, cache, into=None, planes_ok=False, out_dtype=None):
         """``out_dtype``: the type of the branch's output if it is not the compute type (a block that adds
         several branches before the residual sum asks for float32)."""
+        if self.general:
+            return self._forward_general(h, step, cache, out_dtype=out_dtype)
         nh, nkv, dh, dv = self.heads, self.kv_heads, self.padded_dim, self.value_dim       # (dh: as the kernels see a head)
         plain = self.norm_eps is None and self.q_temp is None       # nothing but a rotation between the product and the cache
         if not plain and self.position.rotary_tables() is not None:

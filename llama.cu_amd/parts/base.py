@@ -151,6 +151,46 @@ class SlotState(CacheNeed):
         return LayerCache(state=torch.zeros((slots,) + tuple(self.shape), dtype=self.dtype, device=device))
 
 
+@dataclass(frozen=True)
+class SeveralNeeds(CacheNeed):
+    """The needs of a mixer that is several mixers side by side, each with a need of its own: at most one of them
+    pages (its pool is the whole's), the others states of fixed size.  The mixers all get the one LayerCache: the
+    pages in ``pages``, a single state in ``state``, and with more than one state the i-th need's as
+    ``more["state<i>"]`` (``state`` is then the first)."""
+    needs: Tuple[CacheNeed, ...]
+
+    def __post_init__(self):
+        if sum(1 for n in self.needs if n.pool() is not None) > 1:
+            raise ValueError("several needs side by side: at most one of them may be pages of keys and values")
+
+    @property
+    def can_truncate(self):
+        return all(n.can_truncate for n in self.needs)
+
+    def pool(self):
+        for n in self.needs:
+            if n.pool() is not None:
+                return n.pool()
+        return None
+
+    def page_bytes(self, page_size: int, elem_size: int) -> int:
+        return sum(n.page_bytes(page_size, elem_size) for n in self.needs)
+
+    def allocate(self, group, num_pages, page_size, slots, dtype, device) -> LayerCache:
+        out = LayerCache()
+        states = 0
+        for i, n in enumerate(self.needs):
+            made = n.allocate(group, num_pages, page_size, slots, dtype, device)
+            if made.pages is not None:
+                out.group, out.pages, out.page_size = made.group, made.pages, made.page_size
+            if made.state is not None:
+                if out.state is None:
+                    out.state = made.state
+                out.more[f"state{i}"] = made.state
+                states += 1
+        return out
+
+
 # ------------------------------------------------------------------ building
 
 
@@ -179,6 +219,14 @@ class ScaledRows:
     eps: float
 
 
+@dataclass
+class NormedRows:
+    """The rows that a block's first norm would make of the residual stream, made already by the block before (in
+    the kernel that added that block's last output to the stream): ``rows [n, width]`` in the compute type.  A
+    block hands these only to a block that says it takes them (``takes_normed_rows``)."""
+    rows: torch.Tensor
+
+
 class Part:
     # Whether a step through this part may be captured into a graph and replayed: true only
     # if all it does is launch work on the current stream whose shape depends on the batch's
@@ -200,11 +248,16 @@ class Part:
     # block: ``ends_in_next_norm``: ``forward(..., next_norm=)`` may end in the norm that follows the block;
     #        ``ends_in_planes`` / ``takes_planes`` / ``takes_scaled_rows`` as above, for its last branch
     #        and its first norm.
+    #        ``hands_over_normed``: ``forward(..., next_norm=)`` adds its last output to the stream itself, runs that
+    #        norm in the same kernel and returns NormedRows; ``takes_normed_rows``: ``pending`` may be NormedRows
+    #        made with its ``first_norm``.
     deferrable = False
     takes_planes = False
     ends_in_norm = False
     ends_in_planes = False
     ends_in_next_norm = False
+    hands_over_normed = False
+    takes_normed_rows = False
 
     def takes_scaled_rows(self, n_rows: int) -> bool:
         return False
@@ -221,6 +274,10 @@ class Part:
     # a rotation, any other change of queries and keys in place, a bias inside the scores.
     def rotary_tables(self):
         return None
+
+    def rotated_dims(self) -> int:
+        """position: how many dims of a head a rotation turns (0: none); known before the tables are made."""
+        return 0
 
     def apply(self, qkv, positions, heads, kv_heads, head_dim) -> None:
         pass

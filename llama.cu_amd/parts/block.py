@@ -17,7 +17,7 @@ from typing import Dict, Optional
 import torch
 
 from ..kernels import ops
-from .base import BuildContext, Part, PartSpec, ScaledRows, SlotState, TensorSpec, make_part, prefixed, register_part
+from .base import BuildContext, NormedRows, Part, PartSpec, ScaledRows, SlotState, TensorSpec, make_part, prefixed, register_part
 from .norm import LayerNorm
 
 
@@ -223,3 +223,90 @@ class ParallelBlock(Part):
 
 
 register_part("block", "parallel", ParallelBlock)
+
+
+class SandwichBlock(Part):
+    """A norm in front of and behind every sublayer: ``x += post1(mixer(norm1(x)))``, then ``x += post2(ffn(norm2(x)))``.
+    The feed-forward (with its two norms) may be missing.  The four norms are RMS norms (a factor per row times a
+    weight per column).  The norm behind a sublayer, the residual sum and the norm in front of the next sublayer are
+    one kernel (``ops.norm_post``), also across the border to the next block where that block takes such rows
+    (``NormedRows``); the stream and the sums are 32-bit."""
+
+    def __init__(self, norm1: PartSpec, mixer: PartSpec, post1: PartSpec, norm2: Optional[PartSpec] = None,
+                 ffn: Optional[PartSpec] = None, post2: Optional[PartSpec] = None):
+        if len({norm2 is None, ffn is None, post2 is None}) != 1:
+            raise ValueError("sandwich block: the feed-forward and its two norms come together or not at all")
+        self.specs = {"norm1": norm1, "mixer": mixer, "post1": post1, "norm2": norm2, "ffn": ffn, "post2": post2}
+        self.norm1 = make_part("norm", norm1)
+        self.mixer = make_part("mixer", mixer)
+        self.post1 = make_part("norm", post1)
+        self.norm2 = make_part("norm", norm2) if norm2 is not None else None
+        self.ffn = make_part("ffn", ffn) if ffn is not None else None
+        self.post2 = make_part("norm", post2) if post2 is not None else None
+        for name in ("norm1", "post1", "norm2", "post2"):
+            part = getattr(self, name)
+            if part is not None and not part.deferrable:
+                raise ValueError(f"sandwich block: {name} must be a norm that is a factor per row times a weight per column")
+        self.graph_safe = all(p.graph_safe for _, p in self._children())
+
+    def _children(self):
+        return [(self.specs[k].name, getattr(self, k)) for k in ("norm1", "mixer", "post1", "norm2", "ffn", "post2")
+                if getattr(self, k) is not None]
+
+    def tensors(self) -> Dict[str, TensorSpec]:
+        out = {}
+        for name, part in self._children():
+            for k, v in part.tensors().items():
+                out[prefixed(name, k)] = v
+        return out
+
+    def load(self, tensors, build: BuildContext) -> None:
+        for name, part in self._children():
+            pre = name + "." if name else ""
+            part.load({k[len(pre):]: v for k, v in tensors.items() if k.startswith(pre)}, build)
+        self.dtype = build.dtype
+
+    def fused_groups(self, dtype, device):
+        out = []
+        for name, part in self._children():
+            out += [(tuple(prefixed(name, n) for n in names), pad) for names, pad in part.fused_groups(dtype, device)]
+        return out
+
+    def cache_need(self):
+        return self.mixer.cache_need()
+
+    def prepare(self, step) -> None:
+        for _, part in self._children():
+            part.prepare(step)
+
+    def decode_splits(self, batch: int, max_ctx_len: int) -> int:
+        return int(self.mixer.decode_splits(batch, max_ctx_len))
+
+    @property
+    def first_norm(self):
+        return self.norm1
+
+    hands_over_normed = True     # forward(..., next_norm=) returns NormedRows
+    takes_normed_rows = True     # pending may be NormedRows made with norm1
+
+    @property
+    def takes_planes(self) -> bool:
+        return bool(self.norm1.takes_planes)
+
+    def forward(self, x: torch.Tensor, pending, step, cache, next_norm=None, planes_ok=False):
+        if isinstance(pending, NormedRows):
+            h = pending.rows
+        else:
+            h = self.norm1.forward(x, pending)
+        a = self.mixer.forward(h, step, cache)
+        last, post = a, self.post1
+        if self.ffn is not None:
+            h2 = ops.norm_post(x, a, self.post1.weight32, self.post1.eps, self.norm2.weight32, self.norm2.eps, out_dtype=self.dtype)
+            last, post = self.ffn.forward(h2), self.post2
+        if next_norm is not None:
+            return NormedRows(ops.norm_post(x, last, post.weight32, post.eps, next_norm.weight32, next_norm.eps, out_dtype=self.dtype))
+        ops.norm_post(x, last, post.weight32, post.eps)
+        return None
+
+
+register_part("block", "sandwich", SandwichBlock)

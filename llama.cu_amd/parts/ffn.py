@@ -21,14 +21,18 @@ from .linear import (Weight, library_friendly_rows, linear, linear_into_norm, li
 class SwiGLU(Part):
     graph_safe = True
 
-    def __init__(self, hidden_size: int, intermediate_size: int):
+    # the tensors' names under the part's own; ``names`` replaces any
+    NAMES = {"gate": "gate_proj.weight", "up": "up_proj.weight", "down": "down_proj.weight"}
+
+    def __init__(self, hidden_size: int, intermediate_size: int, names=None):
         self.hidden_size, self.intermediate_size = int(hidden_size), int(intermediate_size)
+        self.names = dict(self.NAMES, **(names or {}))
         self.w_gate_up = self.w_down = None
 
     def tensors(self) -> Dict[str, TensorSpec]:
         d, di = self.hidden_size, self.intermediate_size
-        return {"gate_proj.weight": TensorSpec((di, d)), "up_proj.weight": TensorSpec((di, d)),
-                "down_proj.weight": TensorSpec((d, di))}
+        nm = self.names
+        return {nm["gate"]: TensorSpec((di, d)), nm["up"]: TensorSpec((di, d)), nm["down"]: TensorSpec((d, di))}
 
     def _padded_rows(self, dtype, device) -> int:
         """Rows of each half of the plain gate/up matrix: more than ``intermediate_size`` where the library's
@@ -39,10 +43,10 @@ class SwiGLU(Part):
 
     def fused_groups(self, dtype, device):
         rows = self._padded_rows(dtype, device)
-        return [(("gate_proj.weight", "up_proj.weight"), rows if rows != self.intermediate_size else 0)]
+        return [((self.names["gate"], self.names["up"]), rows if rows != self.intermediate_size else 0)]
 
     def load(self, tensors, build: BuildContext) -> None:
-        g, u = tensors["gate_proj.weight"], tensors["up_proj.weight"]
+        g, u = tensors[self.names["gate"]], tensors[self.names["up"]]
         rows = self.intermediate_size
         if build.dtype == torch.bfloat16 and g.dtype == u.dtype == torch.bfloat16 and g.is_cuda:
             rows = self._padded_rows(build.dtype, g.device)
@@ -53,7 +57,7 @@ class SwiGLU(Part):
             self.w_gate_up = Weight(plain, build, packed_from=torch.cat([g, u], dim=0) if build.pack_weights else None, halves=True)
         else:
             self.w_gate_up = Weight(fused_rows([g, u]), build, halves=True)
-        self.w_down = Weight(tensors["down_proj.weight"], build)
+        self.w_down = Weight(tensors[self.names["down"]], build)
         self.dtype = build.dtype
 
     def takes_scaled_rows(self, n_rows: int) -> bool:

@@ -166,6 +166,10 @@ class DecoderModel:
                 kw = {}
                 if follower is not None and norm is not None and layer.ends_in_next_norm and follower.takes_scaled_rows(x.shape[0]):
                     kw["next_norm"] = norm
+                elif i + 1 < len(order) and norm is not None and layer.hands_over_normed and follower.takes_normed_rows \
+                        and norm.deferrable:
+                    # the block adds its last output to the stream and runs the next block's first norm in one kernel
+                    kw["next_norm"] = norm
                 # a block may leave its last product's partial sums to the norm that adds its output,
                 # if that norm takes them: the next block's first, or the final norm when no rows are
                 # gathered before it

@@ -17,17 +17,23 @@ from .base import BuildContext, Part, TensorSpec, register_part
 class RMSNorm(Part):
     graph_safe = True
 
-    def __init__(self, size: int, eps: float):
+    def __init__(self, size: int, eps: float, tensor: str = "weight", one_plus: bool = False):
+        """``tensor``: the weight's name under the part's.  ``one_plus``: the file holds the weight around zero and the
+        factor is ``1 + w``; the sum is made once, at load, in 32-bit, and ``weight`` is the factor."""
         self.size = int(size)
         self.eps = float(eps)
+        self.tensor, self.one_plus = str(tensor), bool(one_plus)
         self.weight: Optional[torch.Tensor] = None
         self.dtype = None
 
     def tensors(self) -> Dict[str, TensorSpec]:
-        return {"weight": TensorSpec((self.size,), init="one_plus_normal")}
+        return {self.tensor: TensorSpec((self.size,), init="normal" if self.one_plus else "one_plus_normal")}
 
     def load(self, tensors, build: BuildContext) -> None:
-        self.weight = tensors["weight"].contiguous()
+        w = tensors[self.tensor]
+        self.weight = (1.0 + w.float()).contiguous() if self.one_plus else w.contiguous()
+        # the factor in 32-bit, for kernels that take it so (a norm behind a sublayer, ``ops.norm_post``)
+        self.weight32 = self.weight if self.weight.dtype == torch.float32 else self.weight.float().contiguous()
         self.dtype = build.dtype
 
     def forward(self, x: torch.Tensor, delta: Optional[torch.Tensor] = None) -> torch.Tensor:

@@ -46,7 +46,7 @@ class _Tables:
         self.cos, self.sin = cos, sin
 
 
-# The tables depend on (theta, rotated dims, positions, device) alone, so the layers of a model that agree in
+# The tables depend on (theta, rotated dims, positions, device, scaling) alone, so the layers of a model that agree in
 # these share one pair: 32 layers at 131,072 positions would else build and hold 32 x 67 MB.  The table lives as
 # long as a part holds it.
 _tables: "weakref.WeakValueDictionary" = weakref.WeakValueDictionary()
@@ -64,8 +64,12 @@ class Rotary(NoPosition):
     """
 
     def __init__(self, head_dim: int, theta: float, max_positions: int, interleaved: bool = False,
-                 rot_dim: int = 0):
+                 rot_dim: int = 0, scaling_factor: float = 1.0):
+        """``scaling_factor``: linear scaling, every frequency is divided by it (in 32-bit)."""
         self.head_dim = int(head_dim)
+        self.scaling_factor = float(scaling_factor)
+        if not self.scaling_factor > 0:
+            raise ValueError(f"rotary: the scaling factor {scaling_factor} must be positive")
         self.rot_dim = int(rot_dim) if rot_dim else int(head_dim)
         if self.rot_dim % 2 or self.rot_dim > self.head_dim:
             raise ValueError(f"rotary: rot_dim {self.rot_dim} must be even and at most head_dim {self.head_dim}")
@@ -79,12 +83,14 @@ class Rotary(NoPosition):
         # 32-bit throughout, as the reference: theta.powf(-((2 * i) as f32 / dh as f32))
         expo = -(np.float32(2.0) * np.arange(half, dtype=np.float32) / np.float32(self.rot_dim))
         freq = np.power(np.float32(self.theta), expo.astype(np.float32)).astype(np.float32)
+        if self.scaling_factor != 1.0:
+            freq = (freq / np.float32(self.scaling_factor)).astype(np.float32)
         pos = np.arange(self.max_positions, dtype=np.float32)
         ang = (pos[:, None] * freq[None, :]).astype(np.float32).astype(np.float64)   # the 32-bit product
         return np.cos(ang).astype(np.float32), np.sin(ang).astype(np.float32)
 
     def load(self, tensors, build: BuildContext) -> None:
-        key = (self.theta, self.rot_dim, self.max_positions, str(torch.device(build.device)))
+        key = (self.theta, self.rot_dim, self.max_positions, str(torch.device(build.device)), self.scaling_factor)
         tables = _tables.get(key)
         if tables is None:
             cos, sin = self.host_tables()
@@ -95,6 +101,9 @@ class Rotary(NoPosition):
 
     def rotary_tables(self):
         return self.cos, self.sin, self.rot_dim, 1 if self.interleaved else 0
+
+    def rotated_dims(self) -> int:
+        return self.rot_dim
 
 
 class DistanceBias(NoPosition):
