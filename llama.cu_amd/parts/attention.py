@@ -160,6 +160,11 @@ class Attention(Part):
         self.page_size = build.page_size
         self.dtype = build.dtype
 
+    def _matrix_cores(self, page_size: int) -> bool:
+        """Whether the general path's attention runs on the matrix-core kernels (else on the generic one)."""
+        return (self.dtype == torch.bfloat16 and not self.chunk and self.stored_value_dim == self.stored_dim
+                and ops.mfma_attention_refusal(self.dtype, self.heads, self.kv_heads, self.stored_dim, page_size) is None)
+
     def _forward_general(self, h, step, cache, out_dtype=None):
         nh, nkv = self.heads, self.kv_heads
         if not cache.writes:
@@ -174,7 +179,8 @@ class Attention(Part):
                             pairing=pairing, cache=cache.pages, slots=step.slots(cache.group), page_size=page_size)
         out = torch.empty((rows.shape[0], nh * self.stored_value_dim), dtype=self.dtype, device=rows.device)
         ops.paged_attention(q, out, cache.pages, step, cache.group, nh, nkv, self.stored_dim, page_size, self.scale,
-                            self.window, value_dim=self.stored_value_dim, chunk=self.chunk)
+                            self.window, value_dim=self.stored_value_dim, chunk=self.chunk,
+                            force_generic=not self._matrix_cores(page_size))
         if self.head_gate:
             ops.head_gate(out, rows, self.g_off, nh, self.stored_value_dim)
         return linear(out, self.w_o, out_dtype=out_dtype or self.dtype)
@@ -218,9 +224,11 @@ class Attention(Part):
         """The lists by which the matrix-core kernels share out a step that is not all single tokens are made here, on
         the host, and go to the device with the step's arrays; ``forward`` then launches work whose sizes follow from
         the step's sizes alone."""
-        if self.general:
-            return
         page_size = self.own_page_size or self.page_size
+        if self.general:
+            if self._matrix_cores(page_size):
+                ops.plan_attention(step, self.heads, self.kv_heads, self.window)
+            return
         if self.dtype == torch.bfloat16 and (self.position.score_slopes() is None or self.scale > 0) \
                 and self.value_dim == self.padded_dim and ops.mfma_attention_refusal(self.dtype, self.heads, self.kv_heads, self.padded_dim, page_size) is None:
             ops.plan_attention(step, self.heads, self.kv_heads, self.window, biased=self.position.score_slopes() is not None)

@@ -62,18 +62,17 @@ def rotate(x, positions, dims, base, factor=1.0, interleaved=False):
 
 
 def masked_softmax_attention(q, k, v, scale, visible):
-    """q [T, H, d], k [T, G, d], v [T, G, dv]; ``visible(i, j)`` says whether query i sees key j.  -> [T, H, dv]"""
+    """q [T, H, d], k [T, G, d], v [T, G, dv]; ``visible [T, T]`` (bool) says whether query i sees key j (the caller
+    masks the future too).  Query head h uses key/value head h // (H / G).  -> [T, H, dv]"""
     T, H, _ = q.shape
     G = k.shape[1]
     out = np.zeros((T, H, v.shape[2]))
     for h in range(H):
         g = h // (H // G)
-        for i in range(T):
-            js = [j for j in range(i + 1) if visible(i, j)]
-            s = np.array([q[i, h] @ k[j, g] for j in js]) * scale
-            p = np.exp(s - s.max())
-            p /= p.sum()
-            out[i, h] = p @ v[js, g]
+        s = (q[:, h] @ k[:, g].T) * scale
+        s = np.where(visible, s, -np.inf)
+        p = np.exp(s - s.max(axis=1, keepdims=True))
+        out[:, h] = (p / p.sum(axis=1, keepdims=True)) @ v[:, g]
     return out
 
 
@@ -91,7 +90,8 @@ def window_attention(h, w, pre, m):
     q = rotate(q, pos, rot["dims"], rot["base"], factor, interleaved=True)
     k = rotate(k, pos, rot["dims"], rot["base"], factor, interleaved=True)
     size = m["mask"]["size"]
-    o = masked_softmax_attention(q, k, v, m["scale"], lambda i, j: i - j < size)
+    i, j = np.arange(T)[:, None], np.arange(T)[None, :]
+    o = masked_softmax_attention(q, k, v, m["scale"], (j <= i) & (i - j < size))
     return o.reshape(T, H * dv) @ w[pre + "o"].T
 
 
@@ -106,7 +106,8 @@ def chunk_attention(h, w, pre, m, eps):
     q = unit_rms(q, eps) * w[pre + "q.norm"]
     k = unit_rms(k, eps) * w[pre + "k.norm"]
     size = m["mask"]["size"]
-    o = masked_softmax_attention(q, k, v, m["scale"], lambda i, j: i // size == j // size)
+    i, j = np.arange(T)[:, None], np.arange(T)[None, :]
+    o = masked_softmax_attention(q, k, v, m["scale"], (j <= i) & (i // size == j // size))
     gate = sigmoid(h @ w[pre + "g"].T)                       # [T, H]
     o = o * gate[:, :, None]
     return o.reshape(T, H * dv) @ w[pre + "o"].T
@@ -119,10 +120,11 @@ def retention(h, w, pre, m, eps):
     q = linear(h, w, pre + "q").reshape(T, H, d)
     k = linear(h, w, pre + "k").reshape(T, H, d)
     v = linear(h, w, pre + "v").reshape(T, H, dv)
-    rot = m["rot"]
-    pos = np.arange(T)
-    q = rotate(q, pos, rot["dims"], rot["base"])
-    k = rotate(k, pos, rot["dims"], rot["base"]) * d ** -0.5
+    rot = m.get("rot")
+    if rot is not None:
+        pos = np.arange(T)
+        q, k = rotate(q, pos, rot["dims"], rot["base"]), rotate(k, pos, rot["dims"], rot["base"])
+    k = k * d ** -0.5
     o = np.zeros((T, H, dv))
     for hd in range(H):
         S = np.zeros((d, dv))
