@@ -364,6 +364,35 @@ def divasun_config(z, positions):
                                     "max_positions": positions})
 
 
+def lozezen_config(z, positions):
+    """Window attention, two recurrent units and the side-by-side mixer in turn (the order of the design's small models),
+    every layer with the dense feed-forward of the Llama model beside it, so that both have the same feed-forward weights."""
+    from llama_cu_amd.config import LozezenConfig
+    inter = (z["top"] * 2 * z["ff"] // 3 + 127) // 128 * 128
+    d, h, g, w = z["dim"], z["heads"], z["kv_heads"], z["width"]
+    kinds = ["attention", "rglru", "rglru", "parallel"]
+    layers = []
+    for i in range(z["layers"]):
+        kind = kinds[i % len(kinds)]
+        if kind == "attention":
+            m = {"heads": h, "kv_heads": g, "dim": d, "vdim": d, "scale": d ** -0.5, "mask": {"size": 1024},
+                 "rot": {"dims": d // 2, "base": 10000.0, "scaling": {"factor": 8.0}}}
+        elif kind == "rglru":
+            m = {"width": w, "blocks": 16, "conv": 4}
+        else:
+            m = {"left": {"heads": h // 2, "kv_heads": g // 2, "dim": d, "vdim": d, "scale": d ** -0.5, "mask": {"size": 512}},
+                 "right": {"heads": h // 2, "dim": d, "vdim": d, "decay": [1.0 - 2.0 ** (-5 - k % 8) for k in range(h // 2)],
+                           "rot": {"dims": d, "base": 1000000.0}},
+                 "left_scale": 0.6, "right_scale": 0.9}
+        layers.append({"type": kind, "mixer": m, "mlp": {"kind": "dense", "ff": inter}})
+    return LozezenConfig.from_dict({"architecture": "Lozezen", "vocab": z["vocab"], "width": w, "layers": layers, "norm": {"eps": 1e-6},
+                                    "embedding": {"scale": 0.5}, "max_positions": positions})
+
+
+DESIGN_CONFIGS = {"divasun": lambda z, p: divasun_config(z, p), "llama": lambda z, p: llama_like(z, p),
+                  "lozezen": lambda z, p: lozezen_config(z, p)}
+
+
 def llama_like(z, positions):
     from llama_cu_amd.config import LlamaConfig
     inter = (z["top"] * 2 * z["ff"] // 3 + 127) // 128 * 128
@@ -384,8 +413,8 @@ def run_designs(args):
         from llama_cu_amd.engine.runner import ModelRunner
         design, size, what = args.designs_one.split(":")
         z = DESIGN_SIZES[size]
-        cfg = divasun_config(z, 4096) if design == "divasun" else llama_like(z, 4096)
-        vocab = cfg.vocab if design == "divasun" else cfg.vocab_size
+        cfg = DESIGN_CONFIGS[design](z, 4096)
+        vocab = cfg.vocab_size if design == "llama" else cfg.vocab
         runner = ModelRunner.from_config(cfg, 0, dtype=args.dtype, page_size=args.page_size, max_tokens=64 * 1024, max_seqs=66,
                                          max_batch_tokens=PREFILL_TOKENS, use_graphs=False)
         rng = random.Random(0)
@@ -407,14 +436,15 @@ def run_designs(args):
     steps, warmup = min(args.steps, 32), min(args.warmup, 8)
     rows = []
     for name, z in DESIGN_SIZES.items():
-        for design, cfg in (("divasun", divasun_config(z, positions)), ("llama", llama_like(z, positions))):
+        for design in args.designs.split(","):
+            cfg = DESIGN_CONFIGS[design](z, positions)
             rng = random.Random(0)
             biggest = 64
             per_req = prompt + steps + warmup + 2 * biggest + 72
             engine = Engine.from_config(cfg, seed=0, dtype=args.dtype, page_size=page,
                                         max_tokens=biggest * ((per_req + page - 1) // page * page) + PREFILL_TOKENS + page,
                                         max_seqs=biggest + 2, max_batch_tokens=PREFILL_TOKENS, prefill_chunk=PREFILL_TOKENS)
-            vocab = cfg.vocab if design == "divasun" else cfg.vocab_size
+            vocab = cfg.vocab_size if design == "llama" else cfg.vocab
             shim = type("V", (), {"vocab_size": vocab})
             pt = run_prefill(engine, shim, rng, sync)
             row = {"size": name, "design": design, "prefill_tok_s": round(PREFILL_TOKENS / pt, 1), "prefill_ms": round(pt * 1e3, 3)}
@@ -427,7 +457,7 @@ def run_designs(args):
             del engine
             gc.collect()
             torch.cuda.empty_cache()
-    print(json.dumps({"metric": "prefill and decode throughput of two designs at equal layer sizes", "unit": "tok/s", "n_gpus": 1,
+    print(json.dumps({"metric": "prefill and decode throughput of designs at equal layer sizes", "unit": "tok/s", "n_gpus": 1,
                       "dtype": "bf16" if args.dtype == "bfloat16" else "f32", "data": "synthetic", "steps": steps, "warmup": warmup,
                       "sizes": DESIGN_SIZES, "rows": rows}), flush=True)
     return 0
@@ -486,8 +516,11 @@ def main() -> int:
                          "scheduler (the workload that goes with --shape llama2-7b --batch 64); arrivals: --batch requests "
                          "decode while a prompt of 16 tokens arrives every second step (host time and the GPU's busy "
                          "fraction per kind of step)")
+    ap.add_argument("--designs", default="divasun,llama", metavar="NAMES",
+                    help="with --workload designs: which designs are measured side by side, of divasun, lozezen and llama "
+                         "(default: divasun,llama)")
     ap.add_argument("--designs-one", metavar="DESIGN:SIZE:WHAT", default=None,
-                    help="with --workload designs, for a profiler: only DESIGN (divasun or llama) at SIZE (w2048, w4096), and "
+                    help="with --workload designs, for a profiler: only DESIGN (divasun, lozezen or llama) at SIZE (w2048, w4096), and "
                          "only WHAT: 'prefill' (three steps of 2,048 tokens) or a number of requests that decode ten steps over "
                          "prompts of 512 tokens; steps are launched one kernel at a time, not replayed from graphs")
     ap.add_argument("--no-points", action="store_true", help="skip decoding at batch 1 and 64, the prefill and the check")

@@ -33,6 +33,14 @@
 #include "common.h"
 #include "kv_layout.h"
 
+// The first key that the query at position p sees.  window > 0: the last `window` keys; window < 0: the keys of p's own
+// chunk of -window positions, chunks counted from position 0; 0: all keys.  It never falls as p grows.
+__device__ __forceinline__ int first_key(int p, int window) {
+    if (window > 0) return p - window + 1 > 0 ? p - window + 1 : 0;
+    if (window < 0) return p - p % (-window);
+    return 0;
+}
+
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
@@ -327,7 +335,7 @@ attention_decode_kernel(const bf16_t *__restrict__ q, int q_stride, bf16_t *__re
     const int rows = (g - 16 * chunk) < 16 ? (g - 16 * chunk) : 16;
     const int token = q_start[r];
     const int p = ctx_len[r] - 1;
-    const int lo = window > 0 ? (p - window + 1 > 0 ? p - window + 1 : 0) : 0;
+    const int lo = first_key(p, window);
     const int head0 = kvh * g + 16 * chunk;
 
     u32x4 qv[1][DH / 32];
@@ -502,7 +510,7 @@ static int launch_decode(const void *q, int q_stride, void *out, int out_stride,
 // What both decode entry points ask of their sizes (the parts' memory apart): LCU_OK or why not.
 static int decode_arguments(int q_stride, int out_stride, int max_pages, int nh, int nkvh, int dh, int page, int window,
                             int n_splits) {
-    if (nh <= 0 || nkvh <= 0 || nh % nkvh || dh <= 0 || page <= 0 || page % 16 || max_pages <= 0 || window < 0 || n_splits < 1 ||
+    if (nh <= 0 || nkvh <= 0 || nh % nkvh || dh <= 0 || page <= 0 || page % 16 || max_pages <= 0 || n_splits < 1 ||
         n_splits > 65535 || q_stride % 8 || out_stride % 4)
         return LCU_BAD_ARGUMENT;
     if (dh != 32 && dh != 64 && dh != 96 && dh != 128) return LCU_UNSUPPORTED;
@@ -984,13 +992,13 @@ attention_prefill_kernel(const bf16_t *__restrict__ q, int q_stride, bf16_t *__r
         const int last_tok = (tok0 + tokens_per_wave < q_end ? tok0 + tokens_per_wave : q_end) - 1;
         p_max = ctx - (q_end - last_tok);
         p_min = ctx - (q_end - tok0);
-        lo_min = window > 0 && p_min - window + 1 > 0 ? p_min - window + 1 : 0;
-        lo_max = window > 0 && p_max - window + 1 > 0 ? p_max - window + 1 : 0;
+        lo_min = first_key(p_min, window);
+        lo_max = first_key(p_max, window);
     }
     const int wg_last_tok = (task_tok + PRE_WAVES * tokens_per_wave < q_end ? task_tok + PRE_WAVES * tokens_per_wave : q_end) - 1;
     const int wg_p_max = ctx - (q_end - wg_last_tok);
     const int wg_p_min = ctx - (q_end - task_tok);
-    const int wg_lo_min = window > 0 && wg_p_min - window + 1 > 0 ? wg_p_min - window + 1 : 0;
+    const int wg_lo_min = first_key(wg_p_min, window);
 
     PrefillState<DH> st;
     st.m = -INFINITY;
@@ -1021,7 +1029,7 @@ attention_prefill_kernel(const bf16_t *__restrict__ q, int q_stride, bf16_t *__r
     }
     stage_pages<DH, PAGE16>(page_id, tok_in_page, bt, max_pages, page, tile_magic, keys_from(PRE_RING), values_from(PRE_RING), wave);
     const int p_row = tok_row < 0 ? -1 : tok_row + pos_of_tok;
-    const int lo_row = tok_row >= 0 && window > 0 && p_row - window + 1 > 0 ? p_row - window + 1 : 0;
+    const int lo_row = tok_row >= 0 ? first_key(p_row, window) : 0;
     u32x4 kreg[DH / 16], vreg[2 * (DH / 32)];
     u32x4 pb[2] = {u32x4{0u, 0u, 0u, 0u}, u32x4{0u, 0u, 0u, 0u}};
     wait_loads<(PRE_RING - 1) * (DH / 32)>();
@@ -1161,7 +1169,7 @@ LCU_API int lcu_attention_prefill_bf16(const void *q, int q_stride, void *out, i
 #endif
     if ((unsigned long long)kv_page_elems(nkvh, dh, page) * 2ull >= (1ull << 31)) return LCU_UNSUPPORTED;
     if (cache_pages <= 0 || tasks_per_wg < 1 || lcu_attention_prefill_tokens_per_task(nh, nkvh) == 0 || page <= 0 || page % 16 || max_pages <= 0 ||
-        window < 0 || q_stride % 8 || out_stride % 4 || nkvh * ((nh / nkvh + 15) / 16) > 65535)
+        q_stride % 8 || out_stride % 4 || nkvh * ((nh / nkvh + 15) / 16) > 65535)
         return LCU_BAD_ARGUMENT;
 #define GO(D) return launch_prefill<D>(q, q_stride, out, out_stride, cache, cache_pages, block_table, max_pages, q_start, ctx_len, task_req, task_tok0, n_tasks, n_tasks_dev, tasks_per_wg, nh, nkvh, page, scale, window, stream BIAS_ARGS)
     if (dh == 128) GO(128);

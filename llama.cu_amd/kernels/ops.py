@@ -415,14 +415,14 @@ def cut_into_tasks(q_lens, ctx_lens, tokens_per_task: int, skip_single: bool = F
     waiting for them.  (Against all tasks longest first: 60.4 -> 57.8 us for 2,048 tokens over 2k keys, 251.6 ->
     242.7 us over 8k; a long and a short one in turns, or as one workgroup's two tasks, was slower.)  ``skip_single``:
     requests that feed one token get no task (they go to the decode kernel).  ``window``: a task of a layer with a
-    window walks no more keys than its tokens and the window."""
+    window (or, negative, with chunks of so many positions) walks no more keys than its tokens and the window."""
     tasks = []
     start = 0
     for r, n in enumerate(q_lens):
         for t in range(0, n if not (skip_single and n == 1) else 0, tokens_per_task):
             keys = ctx_lens[r] - n + min(t + tokens_per_task, n)        # keys the task's last token sees
-            if window > 0:
-                keys = min(keys, window + tokens_per_task)
+            if window:                  # (negative: chunks of so many positions)
+                keys = min(keys, abs(window) + tokens_per_task)
             tasks.append((-keys, r, start + t))
         start += n
     tasks.sort()
@@ -561,19 +561,23 @@ def paged_attention(q: torch.Tensor, out: torch.Tensor, cache: torch.Tensor, ste
                     chunk: int = 0) -> torch.Tensor:
     """Attention for the batch ``step`` (an engine.batch.StepContext) over cache group
     ``group``: picks the kernel for the batch's shape and type.  ``chunk``: keys of the query's own chunk of so many
-    positions only (the generic kernel).  With a bias inside the scores
+    positions only (the matrix-core kernels take it as a negative window).  With a bias inside the scores
     (``head_slopes``) the matrix-core kernels are those of the second library, which need a positive scale."""
     bt = step.block_table(group)
     if head_slopes is not None:
         _gpu(head_slopes)
         if head_slopes.dtype != torch.float32 or head_slopes.shape != (n_heads,) or not head_slopes.is_contiguous():
             raise KernelError(f"attention: head_slopes must be contiguous float32 [{n_heads}]")
-    if force_generic or chunk or (head_slopes is not None and not scale > 0) or (value_dim and value_dim != head_dim) \
+    if chunk and window:
+        raise KernelError("attention: a window and chunks together are not supported")
+    if force_generic or (head_slopes is not None and not scale > 0) or (value_dim and value_dim != head_dim) \
             or not mfma_attention_supported(q, n_heads, n_kv_heads, head_dim, page_size):
         return paged_attention_generic(q, out, cache, bt, step.q_start, step.ctx_len, step.req_of_token, n_heads,
                                        n_kv_heads, head_dim, page_size, scale, window, head_slopes, value_dim, chunk)
     n = _attention_args(q, out, cache, bt, step.q_start, step.ctx_len, step.req_of_token, n_heads, n_kv_heads, head_dim,
                         page_size)
+    if chunk:
+        window = -int(chunk)
     if step.decode_only:
         splits = step.attn_splits or decode_splits(step.n_req, n_heads, n_kv_heads, step.max_ctx_len)
         # the workgroups start in the order of the requests' list: the requests with the most keys first, where the

@@ -153,16 +153,28 @@ class Attention(Part):
         if self.head_norm_eps is not None:
             self.q_head_norm = tensors[nm["q_head_norm"]].float().contiguous()
             self.k_head_norm = tensors[nm["k_head_norm"]].float().contiguous()
-        self.w_o = Weight(tensors[nm["o"]], build)
+        self.page_size = build.page_size
+        self.dtype = build.dtype
+        # bfloat16: where a head size of the matrix-core kernels holds both the keys' and the values', both are stored
+        # at that size, filled up with dims of zeros (the output matrix gets columns of zeros for the values' zeros)
+        w_o = tensors[nm["o"]]
+        if build.dtype == torch.bfloat16:
+            for size in (32, 64, 96, 128):
+                if size >= max(dh, dv) and ops.mfma_attention_refusal(build.dtype, nh, nkv, size, self.own_page_size or build.page_size) is None:
+                    self.stored_dim = self.stored_value_dim = size
+                    if size != dv:
+                        w_o = torch.cat([w_o.reshape(-1, nh, dv), w_o.new_zeros((w_o.shape[0], nh, size - dv))], dim=2).reshape(w_o.shape[0], nh * size)
+                    break
+            else:
+                ops.say_once(f"attention with {nh} heads of {dh} (values {dv}) in {nkv} groups runs on the generic kernel, not on the matrix cores")
+        self.w_o = Weight(w_o.contiguous(), build)
         self.position.load({}, build)
         if type(self.position).apply is not Part.apply or self.position.score_slopes() is not None:
             raise ValueError("attention: the general path takes a rotation or no position encoding")
-        self.page_size = build.page_size
-        self.dtype = build.dtype
 
     def _matrix_cores(self, page_size: int) -> bool:
         """Whether the general path's attention runs on the matrix-core kernels (else on the generic one)."""
-        return (self.dtype == torch.bfloat16 and not self.chunk and self.stored_value_dim == self.stored_dim
+        return (self.dtype == torch.bfloat16 and self.stored_value_dim == self.stored_dim
                 and ops.mfma_attention_refusal(self.dtype, self.heads, self.kv_heads, self.stored_dim, page_size) is None)
 
     def _forward_general(self, h, step, cache, out_dtype=None):
@@ -227,7 +239,7 @@ class Attention(Part):
         page_size = self.own_page_size or self.page_size
         if self.general:
             if self._matrix_cores(page_size):
-                ops.plan_attention(step, self.heads, self.kv_heads, self.window)
+                ops.plan_attention(step, self.heads, self.kv_heads, -self.chunk if self.chunk else self.window)
             return
         if self.dtype == torch.bfloat16 and (self.position.score_slopes() is None or self.scale > 0) \
                 and self.value_dim == self.padded_dim and ops.mfma_attention_refusal(self.dtype, self.heads, self.kv_heads, self.padded_dim, page_size) is None:
