@@ -8,25 +8,31 @@
 // depends on the width and the block size only.
 #include "common.h"
 
-constexpr int NP_THREADS = 256;
-constexpr int NP_KEEP = 8;          // elements of a row that a thread keeps in registers: rows up to 2048 are read once
+constexpr int NP_KEEP = 8;          // elements of a row that a thread keeps in registers: rows up to 8 x the block's threads are read once
 
-template <class TA, class TO>
-__global__ void __launch_bounds__(NP_THREADS)
+// THREADS: 256, or 1024 where a step has few rows (what counts then is how many loads a row has in flight).  All loads of
+// the kept elements go out before anything waits for one.
+template <class TA, class TO, int THREADS>
+__global__ void __launch_bounds__(THREADS)
 norm_post_kernel(float *__restrict__ x, const TA *__restrict__ a, const float *__restrict__ w_post, float eps_post,
                  const float *__restrict__ w_pre, float eps_pre, TO *__restrict__ out, int d) {
     __shared__ float scratch[16];
     float *xr = x + (size_t)blockIdx.x * d;
     const TA *ar = a + (size_t)blockIdx.x * d;
-    float keep[NP_KEEP];
+    float keep[NP_KEEP], xs[NP_KEEP], wp[NP_KEEP], wq[NP_KEEP];
     float acc = 0.f;
 #pragma unroll
     for (int e = 0; e < NP_KEEP; ++e) {
-        const int c = threadIdx.x + e * NP_THREADS;
-        keep[e] = c < d ? to_f32(ar[c]) : 0.f;
-        acc += keep[e] * keep[e];
+        const int c = threadIdx.x + e * THREADS;
+        const bool in = c < d;
+        keep[e] = in ? to_f32(ar[c]) : 0.f;
+        xs[e] = in ? xr[c] : 0.f;
+        wp[e] = in ? w_post[c] : 0.f;
+        wq[e] = (in && w_pre) ? w_pre[c] : 0.f;
     }
-    for (int c = threadIdx.x + NP_KEEP * NP_THREADS; c < d; c += NP_THREADS) {
+#pragma unroll
+    for (int e = 0; e < NP_KEEP; ++e) acc += keep[e] * keep[e];
+    for (int c = threadIdx.x + NP_KEEP * THREADS; c < d; c += THREADS) {
         const float v = to_f32(ar[c]);
         acc += v * v;
     }
@@ -34,14 +40,14 @@ norm_post_kernel(float *__restrict__ x, const TA *__restrict__ a, const float *_
     acc = 0.f;
 #pragma unroll
     for (int e = 0; e < NP_KEEP; ++e) {
-        const int c = threadIdx.x + e * NP_THREADS;
+        const int c = threadIdx.x + e * THREADS;
         if (c < d) {
-            keep[e] = xr[c] + keep[e] * f_post * w_post[c];
+            keep[e] = xs[e] + keep[e] * f_post * wp[e];
             xr[c] = keep[e];
             acc += keep[e] * keep[e];
         }
     }
-    for (int c = threadIdx.x + NP_KEEP * NP_THREADS; c < d; c += NP_THREADS) {
+    for (int c = threadIdx.x + NP_KEEP * THREADS; c < d; c += THREADS) {
         const float v = xr[c] + to_f32(ar[c]) * f_post * w_post[c];
         xr[c] = v;
         acc += v * v;
@@ -51,10 +57,10 @@ norm_post_kernel(float *__restrict__ x, const TA *__restrict__ a, const float *_
     TO *o = out + (size_t)blockIdx.x * d;
 #pragma unroll
     for (int e = 0; e < NP_KEEP; ++e) {
-        const int c = threadIdx.x + e * NP_THREADS;
-        if (c < d) o[c] = from_f32<TO>(keep[e] * f_pre * w_pre[c]);
+        const int c = threadIdx.x + e * THREADS;
+        if (c < d) o[c] = from_f32<TO>(keep[e] * f_pre * wq[e]);
     }
-    for (int c = threadIdx.x + NP_KEEP * NP_THREADS; c < d; c += NP_THREADS)      // (a thread reads what it wrote itself)
+    for (int c = threadIdx.x + NP_KEEP * THREADS; c < d; c += THREADS)      // (a thread reads what it wrote itself)
         o[c] = from_f32<TO>(xr[c] * f_pre * w_pre[c]);
 }
 
@@ -63,8 +69,12 @@ LCU_API int lcu_norm_post(float *x, const void *a, int a_type, const float *w_po
                           float eps_pre, void *out, int out_type, int n, int d, hipStream_t stream) {
     if (n <= 0) return LCU_OK;
     if (d <= 0 || !x || !a || !w_post || (w_pre && !out)) return LCU_BAD_ARGUMENT;
-    dim3 grid(n), block(NP_THREADS);
-#define GO(TA, TO) norm_post_kernel<TA, TO><<<grid, block, 0, stream>>>(x, (const TA *)a, w_post, eps_post, w_pre, eps_pre, (TO *)out, d)
+    // few rows of some width: 1024 threads a row (a row's sums are then added in another order than with 256: a
+    // difference of rounding between steps of few and of many rows)
+    const bool wide = n <= 64 && d >= 1024;
+    dim3 grid(n);
+#define GO(TA, TO) do { if (wide) norm_post_kernel<TA, TO, 1024><<<grid, dim3(1024), 0, stream>>>(x, (const TA *)a, w_post, eps_post, w_pre, eps_pre, (TO *)out, d); \
+                        else norm_post_kernel<TA, TO, 256><<<grid, dim3(256), 0, stream>>>(x, (const TA *)a, w_post, eps_post, w_pre, eps_pre, (TO *)out, d); } while (0)
     if (a_type == LCU_F32 && out_type == LCU_F32) GO(float, float);
     else if (a_type == LCU_F32 && out_type == LCU_BF16) GO(float, bf16_t);
     else if (a_type == LCU_BF16 && out_type == LCU_BF16) GO(bf16_t, bf16_t);

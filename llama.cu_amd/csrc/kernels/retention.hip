@@ -7,8 +7,9 @@
 //
 // The scan: a request's tokens are one chain, but column j of S depends on column j alone, so a workgroup takes a
 // tile of 32 columns of one head of one request and keeps them in registers from the request's first token of the
-// step to its last: eight lanes a column, each with every eighth key channel; the sum over key channels crosses the
-// eight lanes at the end of a token.  q, k (rotated, 32-bit) and v go through LDS, RT_TOK tokens at a time.  The state
+// step to its last: eight lanes a column, each with an eighth of the key channels; the sum over key channels crosses the
+// eight lanes at the end of a token.  q and k are rotated by a parallel kernel first (32-bit); they and v go through
+// LDS, a stage of tokens at a time, the next stage on its way while the waves work through this one.  The state
 // is taken as zero where the request's first token of the step stands at position 0, and is left as the step's
 // last token makes it.  The order of every sum depends on d alone: however a prompt is cut into steps, the same
 // bits come out.
@@ -19,85 +20,120 @@
 constexpr int RT_THREADS = 256;
 constexpr int RT_LANES = 8;                       // lanes that share a column
 constexpr int RT_COLS = RT_THREADS / RT_LANES;    // columns a workgroup
-constexpr int RT_TOK = 16;                        // tokens staged at a time
 
-template <class TI, int DPL>                      // DPL: key channels per lane (d <= 8 * DPL)
+// q and k of every (token, head), rotated, k scaled, 32-bit: qk [n, nh, 2, d].  A thread per (token, head, dim).
+template <class TI>
+__global__ void __launch_bounds__(256)
+retention_prep_kernel(const TI *__restrict__ rows, int row_stride, int q_off, int k_off, const int *__restrict__ positions,
+                      const float *__restrict__ cos_t, const float *__restrict__ sin_t, int max_pos, int rot_dim, int pairing,
+                      float k_scale, float *__restrict__ qk, int nh, int d) {
+    const int t = blockIdx.x;
+    const TI *row = rows + (size_t)t * row_stride;
+    const int half = rot_dim / 2;
+    const int pos = cos_t ? positions[t] : 0;
+    for (int w = blockIdx.y * blockDim.x + threadIdx.x; w < nh * d; w += gridDim.y * blockDim.x) {
+        const int h = w / d, i = w % d;
+        float qv = to_f32(row[q_off + w]), kv = to_f32(row[k_off + w]);
+        if (cos_t && i < rot_dim) {
+            int pi, partner;
+            bool first;                                   // whether i is the pair's first dim
+            if (pairing == 0) { first = i < half; pi = first ? i : i - half; partner = first ? i + half : i - half; }
+            else { first = (i & 1) == 0; pi = i >> 1; partner = i ^ 1; }
+            const float qp = to_f32(row[q_off + h * d + partner]), kp = to_f32(row[k_off + h * d + partner]);
+            float c = __uint_as_float(0x7fc00000u), sn = c;        // a position outside the table gives NaN
+            if (pos >= 0 && pos < max_pos) { c = cos_t[(size_t)pos * half + pi]; sn = sin_t[(size_t)pos * half + pi]; }
+            float ra, rb;
+            if (first) { rotate_pair(qv, qp, c, sn, ra, rb); qv = ra; rotate_pair(kv, kp, c, sn, ra, rb); kv = ra; }
+            else { rotate_pair(qp, qv, c, sn, ra, rb); qv = rb; rotate_pair(kp, kv, c, sn, ra, rb); kv = rb; }
+        }
+        float *o = qk + ((size_t)t * nh + h) * 2 * d;
+        o[i] = qv;
+        o[d + i] = kv * k_scale;
+    }
+}
+
+// The scan.  DPL: key channels per lane (d <= 8 * DPL), a lane's channels neighbours; TOK: tokens staged at a time.  Two
+// buffers in LDS: while the waves work through one, every thread holds the next tokens' share in registers (loaded
+// before the work began) and writes it into the other afterwards: one barrier a stage.
+template <class TI, int DPL, int TOK>
 __global__ void __launch_bounds__(RT_THREADS)
-retention_scan_kernel(const TI *__restrict__ rows, int row_stride, int q_off, int k_off, int v_off,
-                      const int *__restrict__ positions, const float *__restrict__ cos_t, const float *__restrict__ sin_t,
-                      int max_pos, int rot_dim, int pairing, float k_scale, const float *__restrict__ decay,
-                      float *__restrict__ state, float *__restrict__ o_out, const int *__restrict__ q_start,
-                      const int *__restrict__ ctx_len, const int *__restrict__ state_slot, int nh, int d, int dv) {
+retention_scan_kernel(const TI *__restrict__ rows, int row_stride, int v_off, const float *__restrict__ qk,
+                      const float *__restrict__ decay, float *__restrict__ state, float *__restrict__ o_out,
+                      const int *__restrict__ q_start, const int *__restrict__ ctx_len, const int *__restrict__ state_slot,
+                      int nh, int d, int dv) {
     constexpr int D = 8 * DPL;
-    __shared__ float qs[RT_TOK][D], ks[RT_TOK][D], vs[RT_TOK][RT_COLS];
+    constexpr int STAGE = TOK * (2 * D + RT_COLS);                 // floats of a stage: per token q, k, and the tile of v
+    constexpr int PER = (STAGE + RT_THREADS - 1) / RT_THREADS;     // of which a thread moves so many
+    __shared__ __attribute__((aligned(16))) float lds[2][STAGE];
     const int r = blockIdx.z, h = blockIdx.y, col0 = blockIdx.x * RT_COLS;
     const int t0 = q_start[r], t1 = q_start[r + 1];
     if (t1 <= t0) return;
     const int first_pos = ctx_len[r] - (t1 - t0);
-    const int sub = threadIdx.x % RT_LANES, col = col0 + threadIdx.x / RT_LANES;
+    const int sub = threadIdx.x % RT_LANES, cg = threadIdx.x / RT_LANES, col = col0 + cg;
     const bool live = col < dv;
     float *S = state + ((size_t)state_slot[r] * nh + h) * (size_t)d * dv;
     const float g = decay[h];
     float s[DPL];
 #pragma unroll
     for (int e = 0; e < DPL; ++e) {
-        const int i = sub + RT_LANES * e;
+        const int i = sub * DPL + e;
         s[e] = (live && i < d && first_pos > 0) ? S[(size_t)i * dv + col] : 0.f;
     }
-    const int half = rot_dim / 2;
-    for (int base = t0; base < t1; base += RT_TOK) {
-        const int nt = min(RT_TOK, t1 - base);
-        __syncthreads();
-        // stage: pairs of q and k (rotated), the rest of the dims, the tile of v
-        for (int w = threadIdx.x; w < nt * D; w += RT_THREADS) {
-            const int tt = w / D, i = w % D, t = base + tt;
-            const TI *row = rows + (size_t)t * row_stride;
-            float qv = 0.f, kv = 0.f;
-            if (i < d) {
-                qv = to_f32(row[q_off + h * d + i]);
-                kv = to_f32(row[k_off + h * d + i]);
-                if (cos_t && i < rot_dim) {
-                    const int pos = positions[t];
-                    int pi, partner;
-                    bool first;                                   // whether i is the pair's first dim
-                    if (pairing == 0) { first = i < half; pi = first ? i : i - half; partner = first ? i + half : i - half; }
-                    else { first = (i & 1) == 0; pi = i >> 1; partner = i ^ 1; }
-                    const float qp = to_f32(row[q_off + h * d + partner]), kp = to_f32(row[k_off + h * d + partner]);
-                    float c = __uint_as_float(0x7fc00000u), sn = c;
-                    if (pos >= 0 && pos < max_pos) { c = cos_t[(size_t)pos * half + pi]; sn = sin_t[(size_t)pos * half + pi]; }
-                    float ra, rb;
-                    if (first) { rotate_pair(qv, qp, c, sn, ra, rb); qv = ra; rotate_pair(kv, kp, c, sn, ra, rb); kv = ra; }
-                    else { rotate_pair(qp, qv, c, sn, ra, rb); qv = rb; rotate_pair(kp, kv, c, sn, ra, rb); kv = rb; }
-                }
-                kv *= k_scale;
-            }
-            qs[tt][i] = qv;
-            ks[tt][i] = kv;
+    // element w of a stage: token w / (2D + COLS); within it [0, 2D): q then k (dims beyond d zeros), then the v tile
+    auto fetch = [&](int base, int w) -> float {
+        const int tt = w / (2 * D + RT_COLS), x = w % (2 * D + RT_COLS), t = base + tt;
+        if (w >= STAGE || t >= t1) return 0.f;
+        if (x < 2 * D) {
+            const int which = x / D, i = x % D;
+            return i < d ? qk[(((size_t)t * nh + h) * 2 + which) * d + i] : 0.f;
         }
-        for (int w = threadIdx.x; w < nt * RT_COLS; w += RT_THREADS) {
-            const int tt = w / RT_COLS, c = col0 + w % RT_COLS;
-            vs[tt][w % RT_COLS] = c < dv ? to_f32(rows[(size_t)(base + tt) * row_stride + v_off + h * dv + c]) : 0.f;
+        const int c = col0 + x - 2 * D;
+        return c < dv ? to_f32(rows[(size_t)t * row_stride + v_off + h * dv + c]) : 0.f;
+    };
+    float next[PER];
+#pragma unroll
+    for (int k = 0; k < PER; ++k) next[k] = fetch(t0, threadIdx.x + k * RT_THREADS);
+#pragma unroll
+    for (int k = 0; k < PER; ++k)
+        if (threadIdx.x + k * RT_THREADS < STAGE) lds[0][threadIdx.x + k * RT_THREADS] = next[k];
+    __syncthreads();
+    int buf = 0;
+    for (int base = t0; base < t1; base += TOK, buf ^= 1) {
+        const int nt = min(TOK, t1 - base);
+        const bool more = base + TOK < t1;
+        if (more) {
+#pragma unroll
+            for (int k = 0; k < PER; ++k) next[k] = fetch(base + TOK, threadIdx.x + k * RT_THREADS);
         }
-        __syncthreads();
+        const float *cur = lds[buf];
         for (int tt = 0; tt < nt; ++tt) {
-            const float v = vs[tt][threadIdx.x / RT_LANES];
+            const float *qs = cur + tt * (2 * D + RT_COLS), *ks = qs + D;
+            const float v = qs[2 * D + cg];
             float acc = 0.f;
 #pragma unroll
-            for (int e = 0; e < DPL; ++e) {
-                const int i = sub + RT_LANES * e;
-                s[e] = g * s[e] + ks[tt][i] * v;
-                acc += s[e] * qs[tt][i];
+            for (int e4 = 0; e4 < DPL / 4; ++e4) {
+                const float4 k4 = *(const float4 *)(ks + sub * DPL + 4 * e4), q4 = *(const float4 *)(qs + sub * DPL + 4 * e4);
+                s[4 * e4 + 0] = g * s[4 * e4 + 0] + k4.x * v; acc += s[4 * e4 + 0] * q4.x;
+                s[4 * e4 + 1] = g * s[4 * e4 + 1] + k4.y * v; acc += s[4 * e4 + 1] * q4.y;
+                s[4 * e4 + 2] = g * s[4 * e4 + 2] + k4.z * v; acc += s[4 * e4 + 2] * q4.z;
+                s[4 * e4 + 3] = g * s[4 * e4 + 3] + k4.w * v; acc += s[4 * e4 + 3] * q4.w;
             }
             acc += __shfl_xor(acc, 1, WAVE);
             acc += __shfl_xor(acc, 2, WAVE);
             acc += __shfl_xor(acc, 4, WAVE);
             if (sub == 0 && live) o_out[(size_t)(base + tt) * nh * dv + (size_t)h * dv + col] = acc;
         }
+        if (more) {
+#pragma unroll
+            for (int k = 0; k < PER; ++k)
+                if (threadIdx.x + k * RT_THREADS < STAGE) lds[buf ^ 1][threadIdx.x + k * RT_THREADS] = next[k];
+        }
+        __syncthreads();
     }
     if (live) {
 #pragma unroll
         for (int e = 0; e < DPL; ++e) {
-            const int i = sub + RT_LANES * e;
+            const int i = sub * DPL + e;
             if (i < d) S[(size_t)i * dv + col] = s[e];
         }
     }
@@ -120,23 +156,33 @@ retention_out_kernel(const float *__restrict__ o, const TG *__restrict__ gate, i
 }
 
 // rows: [n, row_stride] of in_type with q (nh * d) at q_off, k at k_off, v (nh * dv) at v_off and the gate (nh * dv)
-// at g_off.  decay: float32 [nh].  state: float32 [slots, nh, d, dv].  o: float32 scratch [n, nh * dv].
+// at g_off.  decay: float32 [nh].  state: float32 [slots, nh, d, dv].  qk: float32 scratch [n, nh, 2, d]; o: float32
+// scratch [n, nh * dv].
 // out: [n, nh * dv] of out_type.  cos_t / sin_t may be null (no rotation).
 LCU_API int lcu_retention(const void *rows, int in_type, int row_stride, int q_off, int k_off, int v_off, int g_off,
                           const int *positions, const float *cos_t, const float *sin_t, int max_pos, int rot_dim, int pairing,
-                          float k_scale, const float *decay, float *state, float *o, void *out, int out_type,
+                          float k_scale, const float *decay, float *state, float *qk, float *o, void *out, int out_type,
                           const int *q_start, const int *ctx_len, const int *state_slot, int n, int n_req, int nh, int d,
                           int dv, float eps, hipStream_t stream) {
     if (n <= 0 || n_req <= 0) return LCU_OK;
     if (nh <= 0 || d <= 0 || d > 256 || dv <= 0 || rot_dim < 0 || rot_dim % 2 || rot_dim > d || (pairing != 0 && pairing != 1) ||
-        !rows || !decay || !state || !o || !out || (cos_t && (!sin_t || !positions)) || nh > 65535 || n_req > 65535)
+        !rows || !decay || !state || !qk || !o || !out || (cos_t && (!sin_t || !positions)) || nh > 65535 || n_req > 65535)
         return LCU_BAD_ARGUMENT;
+    {
+        dim3 pgrid(n, (nh * d + 1023) / 1024), pblock(256);
+        if (in_type == LCU_F32)
+            retention_prep_kernel<float><<<pgrid, pblock, 0, stream>>>((const float *)rows, row_stride, q_off, k_off, positions, cos_t, sin_t, max_pos, rot_dim, pairing, k_scale, qk, nh, d);
+        else if (in_type == LCU_BF16)
+            retention_prep_kernel<bf16_t><<<pgrid, pblock, 0, stream>>>((const bf16_t *)rows, row_stride, q_off, k_off, positions, cos_t, sin_t, max_pos, rot_dim, pairing, k_scale, qk, nh, d);
+        else
+            return LCU_BAD_ARGUMENT;
+        LCU_LAUNCH_CHECK();
+    }
     dim3 grid((dv + RT_COLS - 1) / RT_COLS, nh, n_req), block(RT_THREADS);
-#define SCAN(TI, DPL) retention_scan_kernel<TI, DPL><<<grid, block, 0, stream>>>((const TI *)rows, row_stride, q_off, k_off, v_off, positions, cos_t, sin_t, max_pos, rot_dim, pairing, k_scale, decay, state, o, q_start, ctx_len, state_slot, nh, d, dv)
-#define BY_DIM(TI) do { if (d <= 32) SCAN(TI, 4); else if (d <= 64) SCAN(TI, 8); else if (d <= 128) SCAN(TI, 16); else SCAN(TI, 32); } while (0)
+#define SCAN(TI, DPL, TOK) retention_scan_kernel<TI, DPL, TOK><<<grid, block, 0, stream>>>((const TI *)rows, row_stride, v_off, qk, decay, state, o, q_start, ctx_len, state_slot, nh, d, dv)
+#define BY_DIM(TI) do { if (d <= 32) SCAN(TI, 4, 16); else if (d <= 64) SCAN(TI, 8, 16); else if (d <= 128) SCAN(TI, 16, 16); else SCAN(TI, 32, 8); } while (0)
     if (in_type == LCU_F32) BY_DIM(float);
-    else if (in_type == LCU_BF16) BY_DIM(bf16_t);
-    else return LCU_BAD_ARGUMENT;
+    else BY_DIM(bf16_t);
 #undef BY_DIM
 #undef SCAN
     LCU_LAUNCH_CHECK();

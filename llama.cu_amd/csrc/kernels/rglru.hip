@@ -8,83 +8,122 @@
 //
 // Per request the state is [taps, width] floats: rows 0 .. taps-2 the last taps-1 rows of xin (oldest first), row
 // taps-1 the recurrence's S.  It is taken as zero where the request's first token of the step stands at position 0.
-// Three kernels: the convolution (a thread per token and channel), the gates (a workgroup per block of channels and
-// tile of tokens; the block's two matrices are given transposed, [block][in][out], so that the lanes read neighbours),
-// the scan (a thread per request and channel walks the request's tokens, then leaves the state).  sqrt(1 - a^2) is
+// Two kernels: the convolution with the gates (a workgroup per tile of tokens, block of channels and tile of outputs; the
+// block's two matrices are given transposed, [block][in][out], so that the lanes read neighbours), and the scan (a
+// thread per request and channel walks the request's tokens in their order, then leaves the state; the state is read by
+// the first kernel and written by the second alone).  sqrt(1 - a^2) is
 // taken as sqrt(-expm1(2 log a)): no cancellation where a is close to 1.
 #include "common.h"
 
+// xin of channel c at token t (a row of the step), or what stood `m` tokens before the step's first token of the
+// request (from the state: its row taps - 1 - m; zero before the request's start).
 template <class TI>
-__global__ void rglru_conv_kernel(const TI *__restrict__ rows, int row_stride, int x_off, const float *__restrict__ bias,
-                                  const float *__restrict__ conv_w, const float *__restrict__ conv_b,
-                                  const float *__restrict__ state, float *__restrict__ u, const int *__restrict__ q_start,
-                                  const int *__restrict__ ctx_len, const int *__restrict__ req_of_token,
-                                  const int *__restrict__ state_slot, int width, int taps) {
-    const int t = blockIdx.x;
-    const int r = req_of_token[t];
-    const int t0 = q_start[r];
-    const int first_pos = ctx_len[r] - (q_start[r + 1] - t0);
-    const float *st = state + (size_t)state_slot[r] * taps * width;
-    for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < width; c += gridDim.y * blockDim.x) {
-        float acc = conv_b ? conv_b[c] : 0.f;
-        for (int j = 0; j < taps; ++j) {
-            const int back = taps - 1 - j;                       // how many tokens before t
-            float x = 0.f;
-            if (t - back >= t0) x = to_f32(rows[(size_t)(t - back) * row_stride + x_off + c]) + (bias ? bias[x_off + c] : 0.f);
-            else if (first_pos > 0) {
-                // the row that stood (t0 - (t - back)) tokens before the step: the state's last row is the newest
-                const int k = taps - 1 - (t0 - (t - back));
-                if (k >= 0 && first_pos - (t0 - (t - back)) >= 0) x = st[(size_t)k * width + c];
-            }
-            acc += conv_w[(size_t)c * taps + j] * x;
+__device__ __forceinline__ float conv_at(const TI *__restrict__ rows, int row_stride, int x_off, const float *__restrict__ bias,
+                                         const float *__restrict__ conv_w, const float *__restrict__ conv_b,
+                                         const float *__restrict__ st, int t, int t0, int first_pos, int c, int width, int taps) {
+    float acc = conv_b ? conv_b[c] : 0.f;
+    const float bx = bias ? bias[x_off + c] : 0.f;
+    for (int j = 0; j < taps; ++j) {
+        const int back = taps - 1 - j;                       // how many tokens before t
+        float x = 0.f;
+        if (t - back >= t0) x = to_f32(rows[(size_t)(t - back) * row_stride + x_off + c]) + bx;
+        else {
+            const int m = t0 - (t - back);                   // so many tokens before the step
+            if (first_pos - m >= 0) x = st[(size_t)(taps - 1 - m) * width + c];
         }
-        u[(size_t)t * width + c] = acc;
+        acc += conv_w[(size_t)c * taps + j] * x;
     }
+    return acc;
 }
 
 constexpr int RG_TOK = 8;          // tokens a workgroup of the gates kernel takes
+constexpr int RG_OUT = 32;         // output channels a workgroup takes
+constexpr int RG_SLICES = 8;       // parts into which the sum over a block's input channels is cut (one per 32 threads)
 constexpr int RG_MAX_BS = 1024;    // channels of a block (LDS holds RG_TOK rows of them)
 
-__global__ void __launch_bounds__(256)
-rglru_gates_kernel(const float *__restrict__ u, const float *__restrict__ wa_t, const float *__restrict__ wi_t,
+// The convolution and the gates.  A workgroup takes RG_TOK tokens, one block of channels and RG_OUT of its outputs: it
+// makes u for all the block's channels of its tokens (in LDS; workgroups of the same block make the same u), then each
+// of its eight groups of 32 threads sums over an eighth of the input channels, and the eight partial sums are added in
+// a fixed order.  So a decoding step, with few tokens, still has blocks x (bs / 32) workgroups.
+template <class TI>
+__global__ void __launch_bounds__(RG_OUT * RG_SLICES)
+rglru_gates_kernel(const TI *__restrict__ rows, int row_stride, int x_off, const float *__restrict__ bias,
+                   const float *__restrict__ conv_w, const float *__restrict__ conv_b, const float *__restrict__ state,
+                   const float *__restrict__ wa_t, const float *__restrict__ wi_t,
                    const float *__restrict__ ba, const float *__restrict__ bi, const float *__restrict__ lam, float c_exp,
-                   float *__restrict__ a_out, float *__restrict__ gx_out, int n, int width, int bs) {
-    __shared__ float us[RG_TOK][RG_MAX_BS];
-    const int b = blockIdx.y, t0 = blockIdx.x * RG_TOK;
-    const int nt = min(RG_TOK, n - t0);
+                   float *__restrict__ a_out, float *__restrict__ gx_out, const int *__restrict__ q_start,
+                   const int *__restrict__ ctx_len, const int *__restrict__ req_of_token, const int *__restrict__ state_slot,
+                   int n, int width, int bs, int taps) {
+    __shared__ __attribute__((aligned(16))) float us[RG_TOK][RG_MAX_BS];
+    __shared__ float part[RG_SLICES][RG_TOK][2][RG_OUT];
+    const int b = blockIdx.y, tok0 = blockIdx.x * RG_TOK, o0 = blockIdx.z * RG_OUT;
+    const int nt = min(RG_TOK, n - tok0);
     for (int w = threadIdx.x; w < RG_TOK * bs; w += blockDim.x) {
         const int tt = w / bs, i = w % bs;
-        us[tt][i] = tt < nt ? u[(size_t)(t0 + tt) * width + b * bs + i] : 0.f;
+        float u = 0.f;
+        if (tt < nt) {
+            const int t = tok0 + tt, r = req_of_token[t], t0 = q_start[r];
+            const int first_pos = ctx_len[r] - (q_start[r + 1] - t0);
+            u = conv_at(rows, row_stride, x_off, bias, conv_w, conv_b, state + (size_t)state_slot[r] * taps * width, t, t0,
+                        first_pos, b * bs + i, width, taps);
+        }
+        us[tt][i] = u;
     }
     __syncthreads();
-    const float *wa = wa_t + (size_t)b * bs * bs, *wi = wi_t + (size_t)b * bs * bs;
-    for (int o = threadIdx.x; o < bs; o += blockDim.x) {
-        float ra[RG_TOK], ri[RG_TOK];
+    const int og = threadIdx.x % RG_OUT, slice = threadIdx.x / RG_OUT, o = o0 + og;
+    const int per = (bs + RG_SLICES - 1) / RG_SLICES;
+    const int i0 = slice * per, i1 = min(bs, i0 + per);
+    float ra[RG_TOK], ri[RG_TOK];
 #pragma unroll
-        for (int tt = 0; tt < RG_TOK; ++tt) ra[tt] = ri[tt] = 0.f;
-        for (int i = 0; i < bs; ++i) {
-            const float a = wa[(size_t)i * bs + o], g = wi[(size_t)i * bs + o];
+    for (int tt = 0; tt < RG_TOK; ++tt) ra[tt] = ri[tt] = 0.f;
+    if (o < bs) {
+        const float *wa = wa_t + (size_t)b * bs * bs + o, *wi = wi_t + (size_t)b * bs * bs + o;
+        int i = i0;
+        if (per % 4 == 0 && bs % 4 == 0) {
+            for (; i + 4 <= i1; i += 4) {
+                float a[4], g[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) { a[e] = wa[(size_t)(i + e) * bs]; g[e] = wi[(size_t)(i + e) * bs]; }
+#pragma unroll
+                for (int tt = 0; tt < RG_TOK; ++tt) {
+                    const float4 u = *(const float4 *)&us[tt][i];
+                    ra[tt] += a[0] * u.x; ra[tt] += a[1] * u.y; ra[tt] += a[2] * u.z; ra[tt] += a[3] * u.w;
+                    ri[tt] += g[0] * u.x; ri[tt] += g[1] * u.y; ri[tt] += g[2] * u.z; ri[tt] += g[3] * u.w;
+                }
+            }
+        }
+        for (; i < i1; ++i) {
+            const float a = wa[(size_t)i * bs], g = wi[(size_t)i * bs];
 #pragma unroll
             for (int tt = 0; tt < RG_TOK; ++tt) {
                 ra[tt] += a * us[tt][i];
                 ri[tt] += g * us[tt][i];
             }
         }
-        const int c = b * bs + o;
-        const float l = lam[c];
-        const float sp = l > 20.f ? l : log1pf(expf(l));          // softplus
-        const float bias_a = ba[c], bias_i = bi[c];
-#pragma unroll
-        for (int tt = 0; tt < RG_TOK; ++tt) {
-            if (tt >= nt) break;
-            const float r = 1.0f / (1.0f + expf(-(ra[tt] + bias_a)));
-            const float gate = 1.0f / (1.0f + expf(-(ri[tt] + bias_i)));
-            const float log_a = -c_exp * r * sp;
-            const float mult = sqrtf(-expm1f(2.0f * log_a));
-            a_out[(size_t)(t0 + tt) * width + c] = expf(log_a);
-            gx_out[(size_t)(t0 + tt) * width + c] = mult * gate * us[tt][o];
-        }
     }
+#pragma unroll
+    for (int tt = 0; tt < RG_TOK; ++tt) {
+        part[slice][tt][0][og] = ra[tt];
+        part[slice][tt][1][og] = ri[tt];
+    }
+    __syncthreads();
+    const int tt = slice;                                     // eight slices, eight tokens: a thread finishes one token's channel
+    if (o >= bs || tt >= nt) return;
+    float sa = 0.f, si = 0.f;
+#pragma unroll
+    for (int k = 0; k < RG_SLICES; ++k) {
+        sa += part[k][tt][0][og];
+        si += part[k][tt][1][og];
+    }
+    const int c = b * bs + o;
+    const float l = lam[c];
+    const float sp = l > 20.f ? l : log1pf(expf(l));          // softplus
+    const float r = 1.0f / (1.0f + expf(-(sa + ba[c])));
+    const float gate = 1.0f / (1.0f + expf(-(si + bi[c])));
+    const float log_a = -c_exp * r * sp;
+    const float mult = sqrtf(-expm1f(2.0f * log_a));
+    a_out[(size_t)(tok0 + tt) * width + c] = expf(log_a);
+    gx_out[(size_t)(tok0 + tt) * width + c] = mult * gate * us[tt][o];
 }
 
 __device__ __forceinline__ float gelu_tanh(float z) {
@@ -105,7 +144,23 @@ __global__ void rglru_scan_kernel(const TI *__restrict__ rows, int row_stride, i
     float *st = state + (size_t)state_slot[r] * taps * width;
     float S = first_pos > 0 ? st[(size_t)(taps - 1) * width + c] : 0.f;
     const float by = bias ? bias[y_off + c] : 0.f;
-    for (int t = t0; t < t1; ++t) {
+    // eight tokens at a time: their loads go out together, the chain of multiply-adds follows in the tokens' order
+    int t = t0;
+    for (; t + 8 <= t1; t += 8) {
+        float av[8], gv[8], yv[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            av[e] = a[(size_t)(t + e) * width + c];
+            gv[e] = gx[(size_t)(t + e) * width + c];
+            yv[e] = to_f32(rows[(size_t)(t + e) * row_stride + y_off + c]);
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            S = av[e] * S + gv[e];
+            out[(size_t)(t + e) * width + c] = from_f32<T>(S * gelu_tanh(yv[e] + by));
+        }
+    }
+    for (; t < t1; ++t) {
         S = a[(size_t)t * width + c] * S + gx[(size_t)t * width + c];
         const float y = gelu_tanh(to_f32(rows[(size_t)t * row_stride + y_off + c]) + by);
         out[(size_t)t * width + c] = from_f32<T>(S * y);
@@ -130,31 +185,26 @@ __global__ void rglru_scan_kernel(const TI *__restrict__ rows, int row_stride, i
 
 // rows: [n, row_stride] of in_type, yin at y_off and xin at x_off (width each); bias: null or float32 over the row's
 // columns.  conv_w [width, taps], conv_b [width] (may be null), wa_t / wi_t [blocks, bs, bs] transposed ([in][out]),
-// ba / bi / lam [width], all float32.  state: float32 [slots, taps, width].  u, a, gx: float32 scratch [n, width].
+// ba / bi / lam [width], all float32.  state: float32 [slots, taps, width].  a, gx: float32 scratch [n, width].
 // out: [n, width] of out_type.
 LCU_API int lcu_rglru(const void *rows, int in_type, int row_stride, int y_off, int x_off, const float *bias,
                       const float *conv_w, const float *conv_b, const float *wa_t, const float *wi_t, const float *ba,
-                      const float *bi, const float *lam, float c_exp, float *state, float *u, float *a, float *gx, void *out,
+                      const float *bi, const float *lam, float c_exp, float *state, float *a, float *gx, void *out,
                       int out_type, const int *q_start, const int *ctx_len, const int *req_of_token, const int *state_slot,
                       int n, int n_req, int width, int blocks, int taps, hipStream_t stream) {
     if (n <= 0 || n_req <= 0) return LCU_OK;
     if (width <= 0 || blocks <= 0 || width % blocks || width / blocks > RG_MAX_BS || taps < 1 || taps > 16 || n_req > 65535 ||
-        !rows || !conv_w || !wa_t || !wi_t || !ba || !bi || !lam || !state || !u || !a || !gx || !out)
+        !rows || !conv_w || !wa_t || !wi_t || !ba || !bi || !lam || !state || !a || !gx || !out)
         return LCU_BAD_ARGUMENT;
     const int bs = width / blocks;
     {
-        dim3 grid(n, (width + 1023) / 1024 > 0 ? (width + 1023) / 1024 : 1), block(256);
+        dim3 grid((n + RG_TOK - 1) / RG_TOK, blocks, (bs + RG_OUT - 1) / RG_OUT), block(RG_OUT * RG_SLICES);
         if (in_type == LCU_F32)
-            rglru_conv_kernel<float><<<grid, block, 0, stream>>>((const float *)rows, row_stride, x_off, bias, conv_w, conv_b, state, u, q_start, ctx_len, req_of_token, state_slot, width, taps);
+            rglru_gates_kernel<float><<<grid, block, 0, stream>>>((const float *)rows, row_stride, x_off, bias, conv_w, conv_b, state, wa_t, wi_t, ba, bi, lam, c_exp, a, gx, q_start, ctx_len, req_of_token, state_slot, n, width, bs, taps);
         else if (in_type == LCU_BF16)
-            rglru_conv_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t *)rows, row_stride, x_off, bias, conv_w, conv_b, state, u, q_start, ctx_len, req_of_token, state_slot, width, taps);
+            rglru_gates_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t *)rows, row_stride, x_off, bias, conv_w, conv_b, state, wa_t, wi_t, ba, bi, lam, c_exp, a, gx, q_start, ctx_len, req_of_token, state_slot, n, width, bs, taps);
         else
             return LCU_BAD_ARGUMENT;
-        LCU_LAUNCH_CHECK();
-    }
-    {
-        dim3 grid((n + RG_TOK - 1) / RG_TOK, blocks), block(bs >= 256 ? 256 : (bs + 63) / 64 * 64);
-        rglru_gates_kernel<<<grid, block, 0, stream>>>(u, wa_t, wi_t, ba, bi, lam, c_exp, a, gx, n, width, bs);
         LCU_LAUNCH_CHECK();
     }
     {
