@@ -6,27 +6,46 @@
 //   S <- decay[h] * S + k v^T          o = S^T q
 //
 // The scan: a request's tokens are one chain, but column j of S depends on column j alone, so a workgroup takes a
-// tile of 32 columns of one head of one request and keeps them in registers from the request's first token of the
-// step to its last: eight lanes a column, each with an eighth of the key channels; the sum over key channels crosses the
-// eight lanes at the end of a token.  q and k are rotated by a parallel kernel first (32-bit); they and v go through
+// tile of 16 columns of one head of one request and keeps them in registers from the request's first token of the
+// step to its last: sixteen lanes a column, each with a sixteenth of the key channels; the sum over key channels crosses
+// the sixteen lanes after a stage's last token.  q and k are rotated by a parallel kernel first (32-bit); they and v go through
 // LDS, a stage of tokens at a time, the next stage on its way while the waves work through this one.  The state
 // is taken as zero where the request's first token of the step stands at position 0, and is left as the step's
 // last token makes it.  The order of every sum depends on d alone: however a prompt is cut into steps, the same
 // bits come out.
 //
-// The output: each head's o divided by its root mean square (eps, no weight), times silu(gate) (second kernel).
+// o is written [head][token][dv].  The output: each head's o divided by its root mean square (eps, no weight), times silu(gate) (second kernel).
 #include "common.h"
 
 constexpr int RT_THREADS = 256;
-constexpr int RT_LANES = 8;                       // lanes that share a column
+constexpr int RT_LANES = 16;                      // lanes that share a column
 constexpr int RT_COLS = RT_THREADS / RT_LANES;    // columns a workgroup
 
-// q and k of every (token, head), rotated, k scaled, 32-bit: qk [n, nh, 2, d].  A thread per (token, head, dim).
+// Moves between the lanes of a group of sixteen inside the vector unit (no trip through LDS): the neighbour, the lane two
+// away, the mirror image within eight and within sixteen.  After the first two every lane of a quad holds the quad's sum,
+// so the mirror image within eight brings the other quad's, and the one within sixteen the other eight's.
+__device__ __forceinline__ float lane_xor1(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));     // quad_perm [1, 0, 3, 2]
+}
+__device__ __forceinline__ float lane_xor2(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true));     // quad_perm [2, 3, 0, 1]
+}
+__device__ __forceinline__ float lane_mirror8(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x141, 0xF, 0xF, true));    // row_half_mirror
+}
+
+__device__ __forceinline__ float lane_mirror16(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x140, 0xF, 0xF, true));    // row_mirror
+}
+
+// q and k of every (token, head), rotated, k scaled, and v, 32-bit: qkv [nh][n][2 d + dv], a head's tokens one after the
+// other, so that the scan's workgroups, which own a head, each stream a run of memory of their own (with rows of all
+// heads every workgroup would walk the same few rows at the same time, and those lie in few memory channels).
 template <class TI>
 __global__ void __launch_bounds__(256)
-retention_prep_kernel(const TI *__restrict__ rows, int row_stride, int q_off, int k_off, const int *__restrict__ positions,
+retention_prep_kernel(const TI *__restrict__ rows, int row_stride, int q_off, int k_off, int v_off, const int *__restrict__ positions,
                       const float *__restrict__ cos_t, const float *__restrict__ sin_t, int max_pos, int rot_dim, int pairing,
-                      float k_scale, float *__restrict__ qk, int nh, int d) {
+                      float k_scale, float *__restrict__ qk, int n, int nh, int d, int dv) {
     const int t = blockIdx.x;
     const TI *row = rows + (size_t)t * row_stride;
     const int half = rot_dim / 2;
@@ -46,22 +65,24 @@ retention_prep_kernel(const TI *__restrict__ rows, int row_stride, int q_off, in
             if (first) { rotate_pair(qv, qp, c, sn, ra, rb); qv = ra; rotate_pair(kv, kp, c, sn, ra, rb); kv = ra; }
             else { rotate_pair(qp, qv, c, sn, ra, rb); qv = rb; rotate_pair(kp, kv, c, sn, ra, rb); kv = rb; }
         }
-        float *o = qk + ((size_t)t * nh + h) * 2 * d;
+        float *o = qk + ((size_t)h * n + t) * (2 * d + dv);
         o[i] = qv;
         o[d + i] = kv * k_scale;
     }
+    for (int w = blockIdx.y * blockDim.x + threadIdx.x; w < nh * dv; w += gridDim.y * blockDim.x)
+        qk[((size_t)(w / dv) * n + t) * (2 * d + dv) + 2 * d + w % dv] = to_f32(row[v_off + w]);
 }
 
-// The scan.  DPL: key channels per lane (d <= 8 * DPL), a lane's channels neighbours; TOK: tokens staged at a time.  Two
+// The scan.  DPL: key channels per lane (d <= 16 * DPL), a lane's channels neighbours; TOK: tokens staged at a time.  Two
 // buffers in LDS: while the waves work through one, every thread holds the next tokens' share in registers (loaded
 // before the work began) and writes it into the other afterwards: one barrier a stage.
-template <class TI, int DPL, int TOK>
+template <int DPL, int TOK>
 __global__ void __launch_bounds__(RT_THREADS)
-retention_scan_kernel(const TI *__restrict__ rows, int row_stride, int v_off, const float *__restrict__ qk,
+retention_scan_kernel(const float *__restrict__ qk,
                       const float *__restrict__ decay, float *__restrict__ state, float *__restrict__ o_out,
                       const int *__restrict__ q_start, const int *__restrict__ ctx_len, const int *__restrict__ state_slot,
-                      int nh, int d, int dv) {
-    constexpr int D = 8 * DPL;
+                      int n, int nh, int d, int dv) {
+    constexpr int D = RT_LANES * DPL;
     constexpr int STAGE = TOK * (2 * D + RT_COLS);                 // floats of a stage: per token q, k, and the tile of v
     constexpr int PER = (STAGE + RT_THREADS - 1) / RT_THREADS;     // of which a thread moves so many
     __shared__ __attribute__((aligned(16))) float lds[2][STAGE];
@@ -83,12 +104,13 @@ retention_scan_kernel(const TI *__restrict__ rows, int row_stride, int v_off, co
     auto fetch = [&](int base, int w) -> float {
         const int tt = w / (2 * D + RT_COLS), x = w % (2 * D + RT_COLS), t = base + tt;
         if (w >= STAGE || t >= t1) return 0.f;
+        const float *src = qk + ((size_t)h * n + t) * (2 * d + dv);
         if (x < 2 * D) {
             const int which = x / D, i = x % D;
-            return i < d ? qk[(((size_t)t * nh + h) * 2 + which) * d + i] : 0.f;
+            return i < d ? src[which * d + i] : 0.f;
         }
         const int c = col0 + x - 2 * D;
-        return c < dv ? to_f32(rows[(size_t)t * row_stride + v_off + h * dv + c]) : 0.f;
+        return c < dv ? src[2 * d + c] : 0.f;
     };
     float next[PER];
 #pragma unroll
@@ -106,22 +128,33 @@ retention_scan_kernel(const TI *__restrict__ rows, int row_stride, int v_off, co
             for (int k = 0; k < PER; ++k) next[k] = fetch(base + TOK, threadIdx.x + k * RT_THREADS);
         }
         const float *cur = lds[buf];
-        for (int tt = 0; tt < nt; ++tt) {
+        // the stage's tokens one after the other; each token's sum over the key channels is left in eight lanes' shares
+        // and crosses the lanes after the stage's last token, all tokens' at once (nothing in the chain waits for it)
+        float acc[TOK];
+#pragma unroll
+        for (int tt = 0; tt < TOK; ++tt) {
+            // (no branch around a token: beyond the request's last one k and v are zeros and the decay is 1, which leaves S)
+            const float gt = tt < nt ? g : 1.0f;
             const float *qs = cur + tt * (2 * D + RT_COLS), *ks = qs + D;
             const float v = qs[2 * D + cg];
-            float acc = 0.f;
+            acc[tt] = 0.f;
 #pragma unroll
             for (int e4 = 0; e4 < DPL / 4; ++e4) {
                 const float4 k4 = *(const float4 *)(ks + sub * DPL + 4 * e4), q4 = *(const float4 *)(qs + sub * DPL + 4 * e4);
-                s[4 * e4 + 0] = g * s[4 * e4 + 0] + k4.x * v; acc += s[4 * e4 + 0] * q4.x;
-                s[4 * e4 + 1] = g * s[4 * e4 + 1] + k4.y * v; acc += s[4 * e4 + 1] * q4.y;
-                s[4 * e4 + 2] = g * s[4 * e4 + 2] + k4.z * v; acc += s[4 * e4 + 2] * q4.z;
-                s[4 * e4 + 3] = g * s[4 * e4 + 3] + k4.w * v; acc += s[4 * e4 + 3] * q4.w;
+                s[4 * e4 + 0] = gt * s[4 * e4 + 0] + k4.x * v; acc[tt] += s[4 * e4 + 0] * q4.x;
+                s[4 * e4 + 1] = gt * s[4 * e4 + 1] + k4.y * v; acc[tt] += s[4 * e4 + 1] * q4.y;
+                s[4 * e4 + 2] = gt * s[4 * e4 + 2] + k4.z * v; acc[tt] += s[4 * e4 + 2] * q4.z;
+                s[4 * e4 + 3] = gt * s[4 * e4 + 3] + k4.w * v; acc[tt] += s[4 * e4 + 3] * q4.w;
             }
-            acc += __shfl_xor(acc, 1, WAVE);
-            acc += __shfl_xor(acc, 2, WAVE);
-            acc += __shfl_xor(acc, 4, WAVE);
-            if (sub == 0 && live) o_out[(size_t)(base + tt) * nh * dv + (size_t)h * dv + col] = acc;
+        }
+#pragma unroll
+        for (int tt = 0; tt < TOK; ++tt) {
+            float a = acc[tt];
+            a += lane_xor1(a);
+            a += lane_xor2(a);
+            a += lane_mirror8(a);
+            a += lane_mirror16(a);
+            if (tt < nt && sub == 0 && live) o_out[((size_t)h * n + base + tt) * dv + col] = a;
         }
         if (more) {
 #pragma unroll
@@ -143,9 +176,9 @@ retention_scan_kernel(const TI *__restrict__ rows, int row_stride, int v_off, co
 template <class TG, class T>
 __global__ void __launch_bounds__(WAVE)
 retention_out_kernel(const float *__restrict__ o, const TG *__restrict__ gate, int gate_stride, int g_off, T *__restrict__ out,
-                     int nh, int dv, float eps) {
+                     int n, int nh, int dv, float eps) {
     const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
-    const float *orow = o + (size_t)t * nh * dv + (size_t)h * dv;
+    const float *orow = o + ((size_t)h * n + t) * dv;
     float sq = 0.f;
     for (int c = lane; c < dv; c += WAVE) sq += orow[c] * orow[c];
     const float f = rsqrtf(wave_sum(sq) / (float)dv + eps);
@@ -156,8 +189,8 @@ retention_out_kernel(const float *__restrict__ o, const TG *__restrict__ gate, i
 }
 
 // rows: [n, row_stride] of in_type with q (nh * d) at q_off, k at k_off, v (nh * dv) at v_off and the gate (nh * dv)
-// at g_off.  decay: float32 [nh].  state: float32 [slots, nh, d, dv].  qk: float32 scratch [n, nh, 2, d]; o: float32
-// scratch [n, nh * dv].
+// at g_off.  decay: float32 [nh].  state: float32 [slots, nh, d, dv].  qk: float32 scratch [nh, n, 2 d + dv]; o: float32
+// scratch [nh, n, dv].
 // out: [n, nh * dv] of out_type.  cos_t / sin_t may be null (no rotation).
 LCU_API int lcu_retention(const void *rows, int in_type, int row_stride, int q_off, int k_off, int v_off, int g_off,
                           const int *positions, const float *cos_t, const float *sin_t, int max_pos, int rot_dim, int pairing,
@@ -169,25 +202,22 @@ LCU_API int lcu_retention(const void *rows, int in_type, int row_stride, int q_o
         !rows || !decay || !state || !qk || !o || !out || (cos_t && (!sin_t || !positions)) || nh > 65535 || n_req > 65535)
         return LCU_BAD_ARGUMENT;
     {
-        dim3 pgrid(n, (nh * d + 1023) / 1024), pblock(256);
+        dim3 pgrid(n, (nh * (d > dv ? d : dv) + 1023) / 1024), pblock(256);
         if (in_type == LCU_F32)
-            retention_prep_kernel<float><<<pgrid, pblock, 0, stream>>>((const float *)rows, row_stride, q_off, k_off, positions, cos_t, sin_t, max_pos, rot_dim, pairing, k_scale, qk, nh, d);
+            retention_prep_kernel<float><<<pgrid, pblock, 0, stream>>>((const float *)rows, row_stride, q_off, k_off, v_off, positions, cos_t, sin_t, max_pos, rot_dim, pairing, k_scale, qk, n, nh, d, dv);
         else if (in_type == LCU_BF16)
-            retention_prep_kernel<bf16_t><<<pgrid, pblock, 0, stream>>>((const bf16_t *)rows, row_stride, q_off, k_off, positions, cos_t, sin_t, max_pos, rot_dim, pairing, k_scale, qk, nh, d);
+            retention_prep_kernel<bf16_t><<<pgrid, pblock, 0, stream>>>((const bf16_t *)rows, row_stride, q_off, k_off, v_off, positions, cos_t, sin_t, max_pos, rot_dim, pairing, k_scale, qk, n, nh, d, dv);
         else
             return LCU_BAD_ARGUMENT;
         LCU_LAUNCH_CHECK();
     }
     dim3 grid((dv + RT_COLS - 1) / RT_COLS, nh, n_req), block(RT_THREADS);
-#define SCAN(TI, DPL, TOK) retention_scan_kernel<TI, DPL, TOK><<<grid, block, 0, stream>>>((const TI *)rows, row_stride, v_off, qk, decay, state, o, q_start, ctx_len, state_slot, nh, d, dv)
-#define BY_DIM(TI) do { if (d <= 32) SCAN(TI, 4, 16); else if (d <= 64) SCAN(TI, 8, 16); else if (d <= 128) SCAN(TI, 16, 16); else SCAN(TI, 32, 8); } while (0)
-    if (in_type == LCU_F32) BY_DIM(float);
-    else BY_DIM(bf16_t);
-#undef BY_DIM
+#define SCAN(DPL, TOK) retention_scan_kernel<DPL, TOK><<<grid, block, 0, stream>>>(qk, decay, state, o, q_start, ctx_len, state_slot, n, nh, d, dv)
+    if (d <= 64) SCAN(4, 16); else if (d <= 128) SCAN(8, 16); else SCAN(16, 8);
 #undef SCAN
     LCU_LAUNCH_CHECK();
     dim3 ogrid(n, nh), oblock(WAVE);
-#define OUT(TG, T) retention_out_kernel<TG, T><<<ogrid, oblock, 0, stream>>>(o, (const TG *)rows, row_stride, g_off, (T *)out, nh, dv, eps)
+#define OUT(TG, T) retention_out_kernel<TG, T><<<ogrid, oblock, 0, stream>>>(o, (const TG *)rows, row_stride, g_off, (T *)out, n, nh, dv, eps)
     if (in_type == LCU_F32 && out_type == LCU_F32) OUT(float, float);
     else if (in_type == LCU_F32 && out_type == LCU_BF16) OUT(float, bf16_t);
     else if (in_type == LCU_BF16 && out_type == LCU_BF16) OUT(bf16_t, bf16_t);

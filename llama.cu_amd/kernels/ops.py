@@ -1344,7 +1344,7 @@ def retention(rows: torch.Tensor, offsets: Dict[str, int], decay: torch.Tensor, 
             raise KernelError("rotation tables must be two contiguous float32 tensors [max_pos, rot_dim/2]")
         max_pos = cos.shape[0]
     o = torch.empty((n, hv), dtype=torch.float32, device=rows.device)
-    qk = torch.empty((n, heads, 2, key_dim), dtype=torch.float32, device=rows.device)
+    qk = torch.empty((heads, n, 2 * key_dim + value_dim), dtype=torch.float32, device=rows.device)
     out = torch.empty((n, hv), dtype=out_dtype, device=rows.device)
     lib = build.load("retention")
     _check(lib.lcu_retention(_ptr(rows), _type(rows, "retention rows"), rows.stride(0), offsets["q"], offsets["k"], offsets["v"],
@@ -1389,12 +1389,12 @@ def rglru(rows: torch.Tensor, y_off: int, x_off: int, bias: Optional[torch.Tenso
         raise KernelError(f"rglru: state must be contiguous float32 [slots, {taps}, {width}]")
     if n != step.n or max(step.state_slots, default=0) >= state.shape[0]:
         raise KernelError("rglru: the rows are not the step's, or a request's slot lies outside the state")
-    scratch = torch.empty((2, n, width), dtype=torch.float32, device=rows.device)
+    scratch = torch.empty((3, n, (width + 63) // 64 * 64), dtype=torch.float32, device=rows.device)
     out = torch.empty((n, width), dtype=out_dtype, device=rows.device)
     lib = build.load("rglru")
     _check(lib.lcu_rglru(_ptr(rows), _type(rows, "rglru rows"), rows.stride(0), int(y_off), int(x_off), _ptr(bias), _ptr(conv_w),
                          _ptr(conv_b), _ptr(wa_t), _ptr(wi_t), _ptr(ba), _ptr(bi), _ptr(lam), ctypes.c_float(c_exp), _ptr(state),
-                         _ptr(scratch[0]), _ptr(scratch[1]), _ptr(out), _type(out, "rglru out"), _ptr(step.q_start),
+                         _ptr(scratch[0]), _ptr(scratch[1]), _ptr(scratch[2]), _ptr(out), _type(out, "rglru out"), _ptr(step.q_start),
                          _ptr(step.ctx_len), _ptr(step.req_of_token), _ptr(step.state_slot), n, step.n_req, width, blocks, taps,
                          _stream()), "rglru")
     return out

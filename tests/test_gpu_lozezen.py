@@ -275,6 +275,34 @@ def test_the_recurrent_unit_against_the_recurrence_in_any_cut(dtype, width, bloc
     assert torch.equal(got, whole.float().cpu()), "a cut changed the bits"
 
 
+def test_the_recurrent_unit_over_a_long_prompt_cut_into_runs():
+    """A request that feeds many tokens is scanned in several runs at once whose effects are chained: against the
+    recurrence token by token, beside a short request in the same step, and against the same tokens fed in two steps."""
+    from llama_cu_amd.kernels import ops
+    T, width, blocks, taps = 1100, 72, 3, 3
+    bs = width // blocks
+    rows, short = rnd(T, 2 * width, seed=1), rnd(5, 2 * width, seed=2)
+    bias = rnd(2 * width, seed=3, std=0.3)
+    conv_w, conv_b = rnd(width, taps, seed=4, std=0.5), rnd(width, seed=5, std=0.3)
+    wa, wi = rnd(blocks, bs, bs, seed=6, std=2 / math.sqrt(bs)), rnd(blocks, bs, bs, seed=7, std=2 / math.sqrt(bs))
+    ba, bi, lam = rnd(width, seed=8), rnd(width, seed=9), rnd(width, seed=10, std=1.5) - 4.0       # (decays close to 1: a long memory)
+    names = {"y": "y", "x": "x", "conv": "conv", "ra": "ra", "ri": "ri", "lam": "lam", "o": "o"}
+    w = {"y": torch.eye(2 * width)[:width], "y.b": bias[:width], "x": torch.eye(2 * width)[width:], "x.b": bias[width:], "conv": conv_w,
+         "conv.b": conv_b, "ra": wa, "ra.b": ba.view(blocks, bs), "ri": wi, "ri.b": bi.view(blocks, bs), "lam": lam, "o": torch.eye(width)}
+    w = {k: v.double().numpy() for k, v in w.items()}
+    want = P.rglru(rows.double().numpy(), w, "", {"width": width, "blocks": blocks})
+    args = (0, width, bias.cuda(), conv_w.cuda(), conv_b.cuda(), wa.transpose(1, 2).contiguous().cuda(),
+            wi.transpose(1, 2).contiguous().cuda(), ba.cuda(), bi.cuda(), lam.cuda(), 8.0)
+    state = torch.full((2, taps, width), 7.0, device="cuda")
+    both = ops.rglru(torch.cat([short, rows]).cuda(), *args, state, hand_step([5, T], [5, T], [0, 1]), torch.float32)
+    assert_close(both[5:], want, 2e-4, "the long request")
+    state2 = torch.full((2, taps, width), -1.0, device="cuda")
+    first = ops.rglru(rows[:600].contiguous().cuda(), *args, state2, hand_step([600], [600], [1]), torch.float32)
+    second = ops.rglru(rows[600:].contiguous().cuda(), *args, state2, hand_step([T - 600], [T], [1]), torch.float32)
+    assert_close(torch.cat([first, second]), both[5:], 1e-5, "two steps against one")
+    assert_close(state2[1], state[1], 1e-5, "the states after them")
+
+
 # ------------------------------------------------------------------ whole models through the engine
 
 
