@@ -14,7 +14,7 @@
 // last token makes it.  The order of every sum depends on d alone: however a prompt is cut into steps, the same
 // bits come out.
 //
-// o is written [head][token][dv].  The output: each head's o divided by its root mean square (eps, no weight), times silu(gate) (second kernel).
+// o is written [head][tile of 16 columns][token][16].  The output: each head's o divided by its root mean square (eps, no weight), times silu(gate) (second kernel).
 #include "common.h"
 
 constexpr int RT_THREADS = 256;
@@ -76,29 +76,57 @@ retention_prep_kernel(const TI *__restrict__ rows, int row_stride, int q_off, in
 // The scan.  DPL: key channels per lane (d <= 16 * DPL), a lane's channels neighbours; TOK: tokens staged at a time.  Two
 // buffers in LDS: while the waves work through one, every thread holds the next tokens' share in registers (loaded
 // before the work began) and writes it into the other afterwards: one barrier a stage.
-template <int DPL, int TOK>
+//
+// MODE 0: a request's tokens of the step in one chain (requests that feed fewer than RT_LONG tokens).  A request that
+// feeds more is cut into RT_RUNS runs that are walked at once, twice: MODE 1 walks each run from a state of zeros and
+// leaves the run's own sum B (S_end = decay^len * S_start + B) in run_b; retention_chain_kernel then gives every run the
+// state it really starts from (run_in); MODE 2 walks the runs again from there and writes the outputs, the last run the
+// request's state.  (The same recurrence with its sums in another order: the results differ from one chain by rounding.)
+constexpr int RT_RUNS = 8;
+constexpr int RT_LONG = 512;
+
+// how many of the requests before r feed at least RT_LONG tokens: r's place among those in run_b and run_in
+__device__ __forceinline__ int long_index(const int *__restrict__ q_start, int r) {
+    int li = 0;
+    for (int i = 0; i < r; ++i) li += (q_start[i + 1] - q_start[i] >= RT_LONG);
+    return li;
+}
+
+template <int DPL, int TOK, int MODE>
 __global__ void __launch_bounds__(RT_THREADS)
 retention_scan_kernel(const float *__restrict__ qk,
                       const float *__restrict__ decay, float *__restrict__ state, float *__restrict__ o_out,
                       const int *__restrict__ q_start, const int *__restrict__ ctx_len, const int *__restrict__ state_slot,
-                      int n, int nh, int d, int dv) {
+                      float *__restrict__ run_b, const float *__restrict__ run_in, int n, int nh, int d, int dv) {
     constexpr int D = RT_LANES * DPL;
     constexpr int STAGE = TOK * (2 * D + RT_COLS);                 // floats of a stage: per token q, k, and the tile of v
     constexpr int PER = (STAGE + RT_THREADS - 1) / RT_THREADS;     // of which a thread moves so many
     __shared__ __attribute__((aligned(16))) float lds[2][STAGE];
-    const int r = blockIdx.z, h = blockIdx.y, col0 = blockIdx.x * RT_COLS;
-    const int t0 = q_start[r], t1 = q_start[r + 1];
-    if (t1 <= t0) return;
+    const int r = MODE == 0 ? blockIdx.z : blockIdx.z / RT_RUNS, run = MODE == 0 ? 0 : blockIdx.z % RT_RUNS;
+    const int h = blockIdx.y, col0 = blockIdx.x * RT_COLS;
+    int t0 = q_start[r], t1 = q_start[r + 1];
+    if (t1 <= t0 || (MODE != 0) != (t1 - t0 >= RT_LONG)) return;
     const int first_pos = ctx_len[r] - (t1 - t0);
     const int sub = threadIdx.x % RT_LANES, cg = threadIdx.x / RT_LANES, col = col0 + cg;
     const bool live = col < dv;
     float *S = state + ((size_t)state_slot[r] * nh + h) * (size_t)d * dv;
+    size_t run_at = 0;
+    if (MODE != 0) {
+        const int len = (t1 - t0 + RT_RUNS - 1) / RT_RUNS, end = t1;
+        t0 = min(end, t0 + run * len);
+        t1 = min(end, t0 + len);
+        run_at = (((size_t)long_index(q_start, r) * RT_RUNS + run) * nh + h) * (size_t)d * dv;
+    }
     const float g = decay[h];
     float s[DPL];
 #pragma unroll
     for (int e = 0; e < DPL; ++e) {
         const int i = sub * DPL + e;
-        s[e] = (live && i < d && first_pos > 0) ? S[(size_t)i * dv + col] : 0.f;
+        s[e] = 0.f;
+        if (live && i < d) {
+            if (MODE == 0 && first_pos > 0) s[e] = S[(size_t)i * dv + col];
+            if (MODE == 2) s[e] = run_in[run_at + (size_t)i * dv + col];
+        }
     }
     // element w of a stage: token w / (2D + COLS); within it [0, 2D): q then k (dims beyond d zeros), then the v tile
     auto fetch = [&](int base, int w) -> float {
@@ -147,6 +175,10 @@ retention_scan_kernel(const float *__restrict__ qk,
                 s[4 * e4 + 3] = gt * s[4 * e4 + 3] + k4.w * v; acc[tt] += s[4 * e4 + 3] * q4.w;
             }
         }
+        // after the moves every lane of a column's sixteen holds the token's sum: lane `tt` of them keeps token tt's, and
+        // the stage's outputs leave in one store (o is laid out [head][tile of 16 columns][token][16]: a workgroup's
+        // stage is one run of memory)
+        float mine = 0.f;
 #pragma unroll
         for (int tt = 0; tt < TOK; ++tt) {
             float a = acc[tt];
@@ -154,8 +186,10 @@ retention_scan_kernel(const float *__restrict__ qk,
             a += lane_xor2(a);
             a += lane_mirror8(a);
             a += lane_mirror16(a);
-            if (tt < nt && sub == 0 && live) o_out[((size_t)h * n + base + tt) * dv + col] = a;
+            if (sub == tt) mine = a;
         }
+        if (MODE != 1 && sub < nt && live)
+            o_out[(((size_t)h * gridDim.x + blockIdx.x) * n + base + sub) * RT_COLS + cg] = mine;
         if (more) {
 #pragma unroll
             for (int k = 0; k < PER; ++k)
@@ -163,11 +197,43 @@ retention_scan_kernel(const float *__restrict__ qk,
         }
         __syncthreads();
     }
+    if (MODE == 2 && run != RT_RUNS - 1) return;              // the last run's end is the request's
     if (live) {
+        float *dst = MODE == 1 ? run_b + run_at : S;
 #pragma unroll
         for (int e = 0; e < DPL; ++e) {
             const int i = sub * DPL + e;
-            if (i < d) S[(size_t)i * dv + col] = s[e];
+            if (i < d) dst[(size_t)i * dv + col] = s[e];
+        }
+    }
+}
+
+// The state that every run of a long request starts from: run 0 from the request's state (zeros at position 0), run k + 1
+// from decay^len_k * (run k's start) + (run k's own sum).  A workgroup per (request, head), a thread per element.
+__global__ void retention_chain_kernel(const float *__restrict__ decay, const float *__restrict__ state, const float *__restrict__ run_b,
+                                       float *__restrict__ run_in, const int *__restrict__ q_start, const int *__restrict__ ctx_len,
+                                       const int *__restrict__ state_slot, int nh, int d, int dv) {
+    const int r = blockIdx.y, h = blockIdx.x;
+    const int t0 = q_start[r], t1 = q_start[r + 1], q = t1 - t0;
+    if (q < RT_LONG) return;
+    const int first_pos = ctx_len[r] - q;
+    const size_t per = (size_t)d * dv;
+    const float *S = state + ((size_t)state_slot[r] * nh + h) * per;
+    const size_t at = ((size_t)long_index(q_start, r) * RT_RUNS * nh + h) * per;
+    const int len = (q + RT_RUNS - 1) / RT_RUNS;
+    const float g = decay[h];
+    float pw[RT_RUNS];
+#pragma unroll
+    for (int k = 0; k < RT_RUNS; ++k) {
+        const int s0 = min(t1, t0 + k * len), s1 = min(t1, s0 + len);
+        pw[k] = powf(g, (float)(s1 - s0));
+    }
+    for (size_t e = (size_t)blockIdx.z * blockDim.x + threadIdx.x; e < per; e += (size_t)gridDim.z * blockDim.x) {
+        float in = first_pos > 0 ? S[e] : 0.f;
+#pragma unroll
+        for (int k = 0; k < RT_RUNS; ++k) {
+            run_in[at + (size_t)k * nh * per + e] = in;
+            in = pw[k] * in + run_b[at + (size_t)k * nh * per + e];
         }
     }
 }
@@ -178,23 +244,24 @@ __global__ void __launch_bounds__(WAVE)
 retention_out_kernel(const float *__restrict__ o, const TG *__restrict__ gate, int gate_stride, int g_off, T *__restrict__ out,
                      int n, int nh, int dv, float eps) {
     const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
-    const float *orow = o + ((size_t)h * n + t) * dv;
+    const int tiles = (dv + RT_COLS - 1) / RT_COLS;
+    auto at = [&](int c) { return o[(((size_t)h * tiles + c / RT_COLS) * n + t) * RT_COLS + c % RT_COLS]; };
     float sq = 0.f;
-    for (int c = lane; c < dv; c += WAVE) sq += orow[c] * orow[c];
+    for (int c = lane; c < dv; c += WAVE) sq += at(c) * at(c);
     const float f = rsqrtf(wave_sum(sq) / (float)dv + eps);
     for (int c = lane; c < dv; c += WAVE) {
         const float z = to_f32(gate[(size_t)t * gate_stride + g_off + h * dv + c]);
-        out[(size_t)t * nh * dv + (size_t)h * dv + c] = from_f32<T>(orow[c] * f * (z / (1.0f + expf(-z))));
+        out[(size_t)t * nh * dv + (size_t)h * dv + c] = from_f32<T>(at(c) * f * (z / (1.0f + expf(-z))));
     }
 }
 
 // rows: [n, row_stride] of in_type with q (nh * d) at q_off, k at k_off, v (nh * dv) at v_off and the gate (nh * dv)
 // at g_off.  decay: float32 [nh].  state: float32 [slots, nh, d, dv].  qk: float32 scratch [nh, n, 2 d + dv]; o: float32
-// scratch [nh, n, dv].
+// scratch of nh * n * (dv rounded up to 16) floats; runs: float32 scratch of 2 * (n / 512) * 8 * nh * d * dv floats (null if n < 512).
 // out: [n, nh * dv] of out_type.  cos_t / sin_t may be null (no rotation).
 LCU_API int lcu_retention(const void *rows, int in_type, int row_stride, int q_off, int k_off, int v_off, int g_off,
                           const int *positions, const float *cos_t, const float *sin_t, int max_pos, int rot_dim, int pairing,
-                          float k_scale, const float *decay, float *state, float *qk, float *o, void *out, int out_type,
+                          float k_scale, const float *decay, float *state, float *qk, float *o, float *runs, void *out, int out_type,
                           const int *q_start, const int *ctx_len, const int *state_slot, int n, int n_req, int nh, int d,
                           int dv, float eps, hipStream_t stream) {
     if (n <= 0 || n_req <= 0) return LCU_OK;
@@ -212,8 +279,21 @@ LCU_API int lcu_retention(const void *rows, int in_type, int row_stride, int q_o
         LCU_LAUNCH_CHECK();
     }
     dim3 grid((dv + RT_COLS - 1) / RT_COLS, nh, n_req), block(RT_THREADS);
-#define SCAN(DPL, TOK) retention_scan_kernel<DPL, TOK><<<grid, block, 0, stream>>>(qk, decay, state, o, q_start, ctx_len, state_slot, n, nh, d, dv)
-    if (d <= 64) SCAN(4, 16); else if (d <= 128) SCAN(8, 16); else SCAN(16, 8);
+#define SCAN(DPL, TOK, MODE, G) retention_scan_kernel<DPL, TOK, MODE><<<G, block, 0, stream>>>(qk, decay, state, o, q_start, ctx_len, state_slot, runs, runs ? runs + run_floats : nullptr, n, nh, d, dv)
+#define BY_DIM(MODE, G) do { if (d <= 64) SCAN(4, 16, MODE, G); else if (d <= 128) SCAN(8, 16, MODE, G); else SCAN(16, 8, MODE, G); } while (0)
+    const size_t run_floats = (size_t)(n / RT_LONG) * RT_RUNS * nh * d * dv;
+    BY_DIM(0, grid);
+    LCU_LAUNCH_CHECK();
+    if (n >= RT_LONG) {                 // the step may hold requests that feed many tokens: they are walked in runs
+        if (!runs || n_req * RT_RUNS > 65535) return LCU_BAD_ARGUMENT;
+        dim3 rgrid(grid.x, nh, n_req * RT_RUNS);
+        BY_DIM(1, rgrid);
+        LCU_LAUNCH_CHECK();
+        retention_chain_kernel<<<dim3(nh, n_req, (unsigned)((d * dv + 1023) / 1024)), dim3(256), 0, stream>>>(decay, state, runs, runs + run_floats, q_start, ctx_len, state_slot, nh, d, dv);
+        LCU_LAUNCH_CHECK();
+        BY_DIM(2, rgrid);
+    }
+#undef BY_DIM
 #undef SCAN
     LCU_LAUNCH_CHECK();
     dim3 ogrid(n, nh), oblock(WAVE);

@@ -1343,13 +1343,15 @@ def retention(rows: torch.Tensor, offsets: Dict[str, int], decay: torch.Tensor, 
                 or cos.dim() != 2 or cos.shape[1] * 2 != rot_dim or not cos.is_contiguous() or not sin.is_contiguous():
             raise KernelError("rotation tables must be two contiguous float32 tensors [max_pos, rot_dim/2]")
         max_pos = cos.shape[0]
-    o = torch.empty((n, hv), dtype=torch.float32, device=rows.device)
+    o = torch.empty((heads, n, (value_dim + 15) // 16 * 16), dtype=torch.float32, device=rows.device)
     qk = torch.empty((heads, n, 2 * key_dim + value_dim), dtype=torch.float32, device=rows.device)
     out = torch.empty((n, hv), dtype=out_dtype, device=rows.device)
+    # requests that feed 512 tokens or more are walked in 8 runs: each run's own sum, and the state it starts from
+    runs = torch.empty(2 * (n // 512) * 8 * heads * key_dim * value_dim, dtype=torch.float32, device=rows.device) if n >= 512 else None
     lib = build.load("retention")
     _check(lib.lcu_retention(_ptr(rows), _type(rows, "retention rows"), rows.stride(0), offsets["q"], offsets["k"], offsets["v"],
                              offsets["g"], _ptr(step.positions), _ptr(cos), _ptr(sin), max_pos, int(rot_dim), int(pairing),
-                             ctypes.c_float(k_scale), _ptr(decay), _ptr(state), _ptr(qk), _ptr(o), _ptr(out), _type(out, "retention out"),
+                             ctypes.c_float(k_scale), _ptr(decay), _ptr(state), _ptr(qk), _ptr(o), _ptr(runs), _ptr(out), _type(out, "retention out"),
                              _ptr(step.q_start), _ptr(step.ctx_len), _ptr(step.state_slot), n, step.n_req, heads, key_dim,
                              value_dim, ctypes.c_float(eps), _stream()), "retention")
     return out

@@ -275,6 +275,37 @@ def test_the_recurrent_unit_against_the_recurrence_in_any_cut(dtype, width, bloc
     assert torch.equal(got, whole.float().cpu()), "a cut changed the bits"
 
 
+def test_retention_over_a_long_prompt_cut_into_runs():
+    """A request that feeds many tokens is walked in several runs at once, each first from zeros, then from the state
+    that the runs before it leave: against the recurrence token by token, beside a short request in the same step, and
+    against the same tokens fed in two steps (the second from a state that is not zero)."""
+    from llama_cu_amd.kernels import ops
+    T, heads, d, dv, eps = 1100, 2, 24, 40, 1e-5
+    hk, hv = heads * d, heads * dv
+    off = {"q": 0, "k": hk, "v": 2 * hk, "g": 2 * hk + hv}
+    proj, short = rnd(T, 2 * hk + 2 * hv, seed=1), rnd(5, 2 * hk + 2 * hv, seed=2)
+    decay = [0.97, 0.9995]
+    x = proj.double().numpy()
+    q, k = x[:, :hk].reshape(T, heads, d), x[:, hk:2 * hk].reshape(T, heads, d) * 0.2
+    v, g = x[:, 2 * hk:2 * hk + hv].reshape(T, heads, dv), x[:, 2 * hk + hv:]
+    o, S = np.zeros((T, heads, dv)), np.zeros((heads, d, dv))
+    for t in range(T):
+        for h in range(heads):
+            S[h] = decay[h] * S[h] + np.outer(k[t, h], v[t, h])
+            o[t, h] = S[h].T @ q[t, h]
+    want = P.unit_rms(o, eps).reshape(T, hv) * P.silu(g)
+    dec = torch.tensor(decay, dtype=torch.float32).cuda()
+    state = torch.full((2, heads, d, dv), 7.0, device="cuda")
+    both = ops.retention(torch.cat([short, proj]).cuda(), off, dec, state, hand_step([5, T], [5, T], [0, 1]), heads, d, dv, 0.2, eps, torch.float32)
+    assert_close(both[5:], want, 2e-4, "the long request")
+    assert_close(state[1], S, 2e-4, "its state")
+    state2 = torch.full((2, heads, d, dv), -1.0, device="cuda")
+    first = ops.retention(proj[:520].contiguous().cuda(), off, dec, state2, hand_step([520], [520], [1]), heads, d, dv, 0.2, eps, torch.float32)
+    second = ops.retention(proj[520:].contiguous().cuda(), off, dec, state2, hand_step([T - 520], [T], [1]), heads, d, dv, 0.2, eps, torch.float32)
+    assert_close(torch.cat([first, second]), both[5:], 1e-5, "two steps against one")
+    assert_close(state2[1], state[1], 1e-5, "the states after them")
+
+
 def test_the_recurrent_unit_over_a_long_prompt_cut_into_runs():
     """A request that feeds many tokens is scanned in several runs at once whose effects are chained: against the
     recurrence token by token, beside a short request in the same step, and against the same tokens fed in two steps."""
