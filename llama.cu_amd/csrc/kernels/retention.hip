@@ -118,16 +118,21 @@ retention_scan_kernel(const float *__restrict__ qk,
         run_at = (((size_t)long_index(q_start, r) * RT_RUNS + run) * nh + h) * (size_t)d * dv;
     }
     const float g = decay[h];
+    // the tile of the state goes through LDS (the stages' memory, not yet in use): sixteen lanes read the sixteen
+    // neighbouring columns of a row of the state, where the lanes' own elements lie a row apart
     float s[DPL];
-#pragma unroll
-    for (int e = 0; e < DPL; ++e) {
-        const int i = sub * DPL + e;
-        s[e] = 0.f;
-        if (live && i < d) {
-            if (MODE == 0 && first_pos > 0) s[e] = S[(size_t)i * dv + col];
-            if (MODE == 2) s[e] = run_in[run_at + (size_t)i * dv + col];
+    const float *from = MODE == 0 ? (first_pos > 0 ? S : nullptr) : MODE == 2 ? run_in + run_at : nullptr;
+    float *tile = &lds[0][0];                                  // [D][RT_COLS + 1]
+    if (from) {
+        for (int w = threadIdx.x; w < D * RT_COLS; w += RT_THREADS) {
+            const int i = w / RT_COLS, c = w % RT_COLS;
+            tile[i * (RT_COLS + 1) + c] = (i < d && col0 + c < dv) ? from[(size_t)i * dv + col0 + c] : 0.f;
         }
+        __syncthreads();
     }
+#pragma unroll
+    for (int e = 0; e < DPL; ++e) s[e] = from ? tile[(sub * DPL + e) * (RT_COLS + 1) + cg] : 0.f;
+    __syncthreads();
     // element w of a stage: token w / (2D + COLS); within it [0, 2D): q then k (dims beyond d zeros), then the v tile
     auto fetch = [&](int base, int w) -> float {
         const int tt = w / (2 * D + RT_COLS), x = w % (2 * D + RT_COLS), t = base + tt;
@@ -198,12 +203,15 @@ retention_scan_kernel(const float *__restrict__ qk,
         __syncthreads();
     }
     if (MODE == 2 && run != RT_RUNS - 1) return;              // the last run's end is the request's
-    if (live) {
+    {
         float *dst = MODE == 1 ? run_b + run_at : S;
+        float *tile = &lds[0][0];                              // (the last stage's barrier is behind every wave)
 #pragma unroll
-        for (int e = 0; e < DPL; ++e) {
-            const int i = sub * DPL + e;
-            if (i < d) dst[(size_t)i * dv + col] = s[e];
+        for (int e = 0; e < DPL; ++e) tile[(sub * DPL + e) * (RT_COLS + 1) + cg] = s[e];
+        __syncthreads();
+        for (int w = threadIdx.x; w < D * RT_COLS; w += RT_THREADS) {
+            const int i = w / RT_COLS, c = w % RT_COLS;
+            if (i < d && col0 + c < dv) dst[(size_t)i * dv + col0 + c] = tile[i * (RT_COLS + 1) + c];
         }
     }
 }
