@@ -365,28 +365,28 @@ def divasun_config(z, positions):
 
 
 def lozezen_config(z, positions):
-    """Window attention, two recurrent units and the side-by-side mixer in turn (the order of the design's small models),
-    every layer with the dense feed-forward of the Llama model beside it, so that both have the same feed-forward weights."""
+    """A recurrent unit, window attention, a recurrent unit and the side-by-side mixer in turn, every layer with the dense
+    feed-forward of the Llama model beside it, so that both have the same feed-forward weights."""
     from llama_cu_amd.config import LozezenConfig
     inter = (z["top"] * 2 * z["ff"] // 3 + 127) // 128 * 128
     d, h, g, w = z["dim"], z["heads"], z["kv_heads"], z["width"]
-    kinds = ["attention", "rglru", "rglru", "parallel"]
+    kinds = ["rglru", "attention", "rglru", "parallel"]
     layers = []
     for i in range(z["layers"]):
         kind = kinds[i % len(kinds)]
         if kind == "attention":
             m = {"heads": h, "kv_heads": g, "dim": d, "vdim": d, "scale": d ** -0.5, "mask": {"size": 1024},
-                 "rot": {"dims": d // 2, "base": 10000.0, "scaling": {"factor": 8.0}}}
+                 "rot": {"dims": d // 2, "base": 50000.0, "scaling": {"factor": 4.0}}}
         elif kind == "rglru":
             m = {"width": w, "blocks": 16, "conv": 4}
         else:
             m = {"left": {"heads": h // 2, "kv_heads": g // 2, "dim": d, "vdim": d, "scale": d ** -0.5, "mask": {"size": 512}},
-                 "right": {"heads": h // 2, "dim": d, "vdim": d, "decay": [1.0 - 2.0 ** (-5 - k % 8) for k in range(h // 2)],
-                           "rot": {"dims": d, "base": 1000000.0}},
-                 "left_scale": 0.6, "right_scale": 0.9}
+                 "right": {"heads": h // 2, "dim": d, "vdim": d, "decay": [1.0 - 0.04 / (1 + k) for k in range(h // 2)],
+                           "rot": {"dims": d, "base": 200000.0}},
+                 "left_scale": 0.75, "right_scale": 1.25}
         layers.append({"type": kind, "mixer": m, "mlp": {"kind": "dense", "ff": inter}})
-    return LozezenConfig.from_dict({"architecture": "Lozezen", "vocab": z["vocab"], "width": w, "layers": layers, "norm": {"eps": 1e-6},
-                                    "embedding": {"scale": 0.5}, "max_positions": positions})
+    return LozezenConfig.from_dict({"architecture": "Lozezen", "vocab": z["vocab"], "width": w, "layers": layers, "norm": {"eps": 1e-5},
+                                    "embedding": {"scale": 2.0}, "max_positions": positions})
 
 
 DESIGN_CONFIGS = {"divasun": lambda z, p: divasun_config(z, p), "llama": lambda z, p: llama_like(z, p),
