@@ -112,5 +112,25 @@ def test_plain_mechanisms_one_by_one():
     seq = rng.standard_normal((6, 1))
     assert np.allclose(P.causal_conv(seq, cw, np.zeros(1)), seq)
     assert np.allclose(P.causal_conv(seq, np.array([[1.0, 0.0, 0.0]]), np.zeros(1))[2:], seq[:-2])
-    # retention of one head with decay 1 and keys e_0: o_t is the running sum of the values times q_0
     assert np.isclose(P.gelu_tanh(np.array(1.0)), 0.841192, atol=1e-6) and np.isclose(P.softplus(np.array(0.0)), np.log(2.0))
+    # retention of one head with decay 1, keys and queries e_0 (times 1 / sqrt(dim) on the keys): o_t is the running sum
+    # of the values, and its norm and gate follow
+    d, T = 4, 5
+    h = rng.standard_normal((T, d))
+    w = {"q": np.zeros((d, d)), "k": np.zeros((d, d)), "v": np.eye(d), "g": np.eye(d), "o": np.eye(d)}
+    w["q"][0], w["k"][0] = np.ones(d), np.ones(d)                      # q_0 = k_0 = sum of the input, the other channels zero
+    m = {"heads": 1, "dim": d, "vdim": d, "decay": [1.0]}
+    s = h.sum(1)
+    o = np.cumsum((s * d ** -0.5)[:, None] * h, axis=0) * s[:, None]
+    assert np.allclose(P.retention(h, w, "", m, 1e-9), P.unit_rms(o, 1e-9) * P.silu(h))
+
+
+def test_several_needs_join_pages_and_states_and_refuse_two_kinds_of_pages():
+    from llama_cu_amd.parts import PagedKV, SeveralNeeds, SlotState
+    both = SeveralNeeds((SlotState((2, 3), torch.float32), PagedKV(2, 16, window=9), SlotState((5,), torch.float32)))
+    assert both.pool() == (9, 0) and not both.can_truncate and both.page_bytes(16, 2) == 2 * 32 * 16 * 2
+    made = both.allocate(0, 4, 16, 3, torch.bfloat16, "cpu")
+    assert made.pages.shape == (4, 2, 2 * 16 * 16) and made.state.shape == (3, 2, 3)
+    assert made.more["state0"].shape == (3, 2, 3) and made.more["state2"].shape == (3, 5)
+    with pytest.raises(ValueError):
+        SeveralNeeds((PagedKV(1, 8), PagedKV(1, 8, window=4)))
