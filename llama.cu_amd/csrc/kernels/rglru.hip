@@ -35,15 +35,16 @@ __device__ __forceinline__ float conv_at(const TI *__restrict__ rows, int row_st
                                          const float *__restrict__ st, int t, int t0, int first_pos, int c, int width, int taps) {
     float acc = conv_b ? conv_b[c] : 0.f;
     const float bx = bias ? bias[x_off + c] : 0.f;
+    // no branch around a load: both places are read (at indices that exist) and one value is chosen, so that the loads of
+    // all taps, and of the elements that a thread makes one after the other, are in flight together
     for (int j = 0; j < taps; ++j) {
         const int back = taps - 1 - j;                       // how many tokens before t
-        float x = 0.f;
-        if (t - back >= t0) x = to_f32(rows[(size_t)(t - back) * row_stride + x_off + c]) + bx;
-        else {
-            const int m = t0 - (t - back);                   // so many tokens before the step
-            if (first_pos - m >= 0) x = st[(size_t)(taps - 1 - m) * width + c];
-        }
-        acc += conv_w[(size_t)c * taps + j] * x;
+        const bool in_step = t - back >= t0;
+        const int m = in_step ? 1 : t0 - (t - back);         // else: so many tokens before the step
+        const bool in_state = !in_step && first_pos - m >= 0;
+        const float here = to_f32(rows[(size_t)(in_step ? t - back : t) * row_stride + x_off + c]) + bx;
+        const float before = st[(size_t)(in_state ? taps - 1 - m : 0) * width + c];
+        acc += conv_w[(size_t)c * taps + j] * (in_step ? here : in_state ? before : 0.f);
     }
     return acc;
 }
@@ -71,6 +72,7 @@ rglru_gates_kernel(const TI *__restrict__ rows, int row_stride, int x_off, const
     __shared__ float part[RG_SLICES][RG_TOK][2][RG_OUT];
     const int b = blockIdx.y, tok0 = blockIdx.x * RG_TOK, o0 = blockIdx.z * RG_OUT;
     const int nt = min(RG_TOK, n - tok0);
+#pragma unroll 4
     for (int w = threadIdx.x; w < RG_TOK * bs; w += blockDim.x) {
         const int tt = w / bs, i = w % bs;
         float u = 0.f;
@@ -164,6 +166,7 @@ rglru_gates_rows_kernel(const TI *__restrict__ rows, int row_stride, int x_off, 
     const int bs4 = (bs + 3) / 4 * 4;
     const int b = blockIdx.y, tok0 = blockIdx.x * RG_ROWS;
     const int nt = min(RG_ROWS, n - tok0);
+#pragma unroll 4
     for (int w = threadIdx.x; w < RG_ROWS * bs4; w += blockDim.x) {
         const int tt = w / bs4, i = w % bs4;
         float u = 0.f;

@@ -306,11 +306,13 @@ def test_retention_over_a_long_prompt_cut_into_runs():
     assert_close(state2[1], state[1], 1e-5, "the states after them")
 
 
-def test_the_recurrent_unit_over_a_long_prompt_cut_into_runs():
+@pytest.mark.parametrize("width,blocks,taps", [(72, 3, 3), (128, 2, 4), (320, 1, 2)])
+def test_the_recurrent_unit_over_a_long_prompt_cut_into_runs(width, blocks, taps):
     """A request that feeds many tokens is scanned in several runs at once whose effects are chained: against the
-    recurrence token by token, beside a short request in the same step, and against the same tokens fed in two steps."""
+    recurrence token by token, beside a short request in the same step, and against the same tokens fed in two steps.
+    (Blocks of 24, 64 and 320 channels: the last are more than a workgroup's threads.)"""
     from llama_cu_amd.kernels import ops
-    T, width, blocks, taps = 1100, 72, 3, 3
+    T = 1100
     bs = width // blocks
     rows, short = rnd(T, 2 * width, seed=1), rnd(5, 2 * width, seed=2)
     bias = rnd(2 * width, seed=3, std=0.3)
